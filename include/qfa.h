@@ -1,0 +1,124 @@
+/*
+ * qfa.h -- C ABI of libqfa.so: per-token asymmetric INT8 quantizer and INT8-QK^T
+ * flash attention (forward + backward) for AMD MI355X (gfx950).
+ *
+ * Conventions shared by every entry point
+ *   - Every pointer is a DEVICE pointer owned by the caller.  Nothing is allocated,
+ *     freed or retained by the library.
+ *   - Tensors are [B, H, N, D] (batch, heads, tokens, head_dim) with the last axis
+ *     contiguous.  s?b / s?h / s?n are strides in ELEMENTS of the b, h and n axes.
+ *   - Per-token vectors (scale, zero point, row sum, LSE, delta) are dense [B*H*N].
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Work is
+ *     enqueued asynchronously; the call returns as soon as the launches are queued.
+ *   - Return value: 0 = success, < 0 = one of the QFA_E* argument errors (nothing was
+ *     launched), > 0 = the hipError_t of a failed launch.  qfa_last_error() returns a
+ *     thread-local, human readable description of the last failure on this thread.
+ *   - The library keeps no mutable global state; calls from several host threads are safe.
+ *
+ * Reference interface each entry point replaces (paths in yisunlp/quant_flash_attn):
+ * the reference has no FFI; the boundary is the Triton launch made by its Python operators.
+ */
+#ifndef QFA_H_
+#define QFA_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QFA_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* element types of floating-point tensors */
+#define QFA_F32 0
+#define QFA_F16 1
+#define QFA_BF16 2
+
+/* argument errors */
+#define QFA_EINVAL (-1)       /* null pointer, non-positive size, bad dtype code, misaligned pointer/stride */
+#define QFA_EUNSUPPORTED (-2) /* well-formed but not implemented (head_dim, causal with Nq != Nk, ...) */
+
+int qfa_version(void);
+const char *qfa_last_error(void);
+
+/*
+ * Per-token asymmetric INT8 quantization over the last axis.
+ * Replaces the launch of _asymmetric_quant_kernel made by asymmetric_quant_per_token
+ * (asymmetric_quant.py:22-106 kernel, :109-149 wrapper).  For every token row x[0..D):
+ *     scale = (max - min) / 255  (1.0 if that is 0);  zp = clamp(roundf(-128 - min/scale))
+ *     code[d] = clamp(roundf(x[d]/scale + zp))         -- all IEEE binary32, roundf = ties away
+ *   x         [B,H,N,D] of x_dtype (QFA_F32 / QFA_F16 / QFA_BF16), strides sxb,sxh,sxn
+ *   codes     [B,H,N,D] int8, strides scb,sch,scn (the reference uses the input's strides)
+ *   scale_f32 [B*H*N] float: the unrounded scale the codes were computed with
+ *   scale_lp  nullable; [B*H*N] copy of the scale rounded to scale_lp_dtype (QFA_F16/QFA_BF16)
+ *             -- the fp16 scale tensor the reference returns (asymmetric_quant.py:93,128)
+ *   zp        [B*H*N] int8
+ *   rowsum    nullable; [B*H*N] int32 sum of the token's codes (feeds the zero-point
+ *             cross term of qfa_attn_fwd / qfa_attn_bwd; not produced by the reference)
+ *   D in {32, 64, 128, 256}.  x and codes 16-byte aligned, strides multiples of 16 bytes.
+ */
+int qfa_quant_per_token(const void *x, int x_dtype, int8_t *codes, float *scale_f32, void *scale_lp,
+                        int scale_lp_dtype, int8_t *zp, int32_t *rowsum, int64_t B, int64_t H, int64_t N,
+                        int D, int64_t sxb, int64_t sxh, int64_t sxn, int64_t scb, int64_t sch, int64_t scn,
+                        void *stream);
+
+/*
+ * out = (codes - zp) * scale, per token (asymmetric_quant.py:158-160, and the in-kernel
+ * dequantization quant_flash_attn.py:65).  scale_dtype is the element type of `scale`
+ * (QFA_F32 / QFA_F16 / QFA_BF16); out has out_dtype and strides sob,soh,son.
+ */
+int qfa_dequant_per_token(const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp, void *out,
+                          int out_dtype, int64_t B, int64_t H, int64_t N, int D, int64_t scb, int64_t sch,
+                          int64_t scn, int64_t sob, int64_t soh, int64_t son, void *stream);
+
+/*
+ * Attention forward on quantized Q and K:
+ *     S = sm_scale * Q^ K^T,  Q^ = sq*(qc - zq),  K^ = sk*(kc - zk)   [causal: keep col <= row]
+ *     O = softmax(S) V,   LSE = logsumexp(S) (natural log)
+ * QK^T runs on INT8 MFMA with int32 accumulation; the zero points enter through the exact
+ * integer cross term (uses the row sums rq, rk).  Softmax is fp32; P.V is bf16/fp16 MFMA.
+ * Replaces the launch of _attn_fwd_kernel_quantized made by QuantFlashAttention.forward
+ * (quant_flash_attn.py:22-83 kernel, :178-204 wrapper), generalised to a quantized Q,
+ * separate K and V, a causal flag (rule of flash_attn_triton.py:50) and tiled queries.
+ *   qc,kc  int8 [B,H,Nq|Nk,D];  sq,sk float, zq,zk int8, rq,rk int32: dense [B*H*Nq|Nk]
+ *   v, o   [B,H,Nk|Nq,D] of io_dtype (QFA_BF16 or QFA_F16);  lse float [B*H*Nq]
+ *   D in {64, 128}.  causal != 0 requires Nq == Nk.  All tensors 16-byte aligned, strides
+ *   multiples of 16 bytes.
+ */
+int qfa_attn_fwd(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,
+                 const float *sk, const int8_t *zk, const int32_t *rk, const void *v, void *o, float *lse,
+                 int io_dtype, int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D, int64_t sqb, int64_t sqh,
+                 int64_t sqn, int64_t skb, int64_t skh, int64_t skn, int64_t svb, int64_t svh, int64_t svn,
+                 int64_t sob, int64_t soh, int64_t son, float sm_scale, int causal, void *stream);
+
+/*
+ * delta[b,h,n] = sum_d O[b,h,n,d] * dO[b,h,n,d], accumulated in fp32.
+ * Replaces the launch of _bwd_preprocess_kernel (quant_flash_attn.py:87-101, :217-223).
+ * qfa_attn_bwd calls this itself; it is exported for callers that split the backward.
+ */
+int qfa_bwd_delta(const void *o, const void *dout, float *delta, int io_dtype, int64_t B, int64_t H, int64_t N,
+                  int D, int64_t sob, int64_t soh, int64_t son, int64_t sdb, int64_t sdh, int64_t sdn,
+                  void *stream);
+
+/*
+ * Attention backward.  Recomputes P = exp(S - LSE) with the same INT8 score path as the
+ * forward, then   dV = P^T dO,  dP = dO V^T,  dS = P o (dP - delta),
+ *                 dQ = sm_scale dS K^,  dK = sm_scale dS^T Q^      (gradients w.r.t. Q^, K^).
+ * Replaces the launches made by QuantFlashAttention.backward (quant_flash_attn.py:104-166
+ * kernel, :207-237 wrapper); the reference's single dKV tensor is dK + dV (:161).
+ *   delta  float [B*H*Nq] workspace, overwritten.
+ *   dq [B,H,Nq,D], dk, dv [B,H,Nk,D] of io_dtype, strides as given.
+ */
+int qfa_attn_bwd(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,
+                 const float *sk, const int8_t *zk, const int32_t *rk, const void *v, const void *o,
+                 const void *dout, const float *lse, float *delta, void *dq, void *dk, void *dv, int io_dtype,
+                 int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D, int64_t sqb, int64_t sqh, int64_t sqn,
+                 int64_t skb, int64_t skh, int64_t skn, int64_t svb, int64_t svh, int64_t svn, int64_t sob,
+                 int64_t soh, int64_t son, int64_t sdob, int64_t sdoh, int64_t sdon, int64_t sdqb, int64_t sdqh,
+                 int64_t sdqn, int64_t sdkb, int64_t sdkh, int64_t sdkn, int64_t sdvb, int64_t sdvh,
+                 int64_t sdvn, float sm_scale, int causal, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QFA_H_ */

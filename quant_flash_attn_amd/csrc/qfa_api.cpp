@@ -1,0 +1,164 @@
+// C entry points of libqfa.so: argument validation, then dispatch to the kernel launchers.
+// Validation touches no HIP API, so a rejected call works (and is testable) without a GPU.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "qfa_host.h"
+
+namespace qfa {
+
+static thread_local char g_err[512] = "";
+
+int set_error(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char *what) {
+  const hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return 0;
+  set_error((int)e, "%s: launch failed: %s", what, hipGetErrorString(e));
+  return (int)e;
+}
+
+static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static bool is_float_dtype(int d) { return d == QFA_F32 || d == QFA_F16 || d == QFA_BF16; }
+static int elem_size(int d) { return d == QFA_F32 ? 4 : 2; }
+
+// strides (elements) of a [B,H,N,D] tensor with element size `es`: positive, 16-byte multiples,
+// and the token stride must at least span a row
+static bool strides_ok(int64_t sb, int64_t sh, int64_t sn, int D, int es) {
+  if (sb <= 0 || sh <= 0 || sn < D) return false;
+  return (sb * es) % 16 == 0 && (sh * es) % 16 == 0 && (sn * es) % 16 == 0;
+}
+
+}  // namespace qfa
+
+using namespace qfa;
+
+extern "C" {
+
+int qfa_version(void) { return QFA_VERSION; }
+
+const char *qfa_last_error(void) { return g_err; }
+
+int qfa_quant_per_token(const void *x, int x_dtype, int8_t *codes, float *scale_f32, void *scale_lp,
+                        int scale_lp_dtype, int8_t *zp, int32_t *rowsum, int64_t B, int64_t H, int64_t N, int D,
+                        int64_t sxb, int64_t sxh, int64_t sxn, int64_t scb, int64_t sch, int64_t scn, void *stream) {
+  if (!x || !codes || !scale_f32 || !zp) return set_error(QFA_EINVAL, "quant: null x/codes/scale_f32/zp pointer");
+  if (!is_float_dtype(x_dtype)) return set_error(QFA_EINVAL, "quant: x_dtype %d is not QFA_F32/F16/BF16", x_dtype);
+  if (scale_lp && scale_lp_dtype != QFA_F16 && scale_lp_dtype != QFA_BF16)
+    return set_error(QFA_EINVAL, "quant: scale_lp_dtype %d is not QFA_F16/BF16", scale_lp_dtype);
+  if (B <= 0 || H <= 0 || N <= 0) return set_error(QFA_EINVAL, "quant: B, H, N must be positive");
+  if (D != 32 && D != 64 && D != 128 && D != 256)
+    return set_error(QFA_EUNSUPPORTED, "quant: head_dim %d not in {32, 64, 128, 256}", D);
+  if (!aligned16(x) || !aligned16(codes)) return set_error(QFA_EINVAL, "quant: x and codes must be 16-byte aligned");
+  if (!strides_ok(sxb, sxh, sxn, D, elem_size(x_dtype)))
+    return set_error(QFA_EINVAL, "quant: x strides must be positive multiples of 16 bytes, token stride >= D");
+  if (!strides_ok(scb, sch, scn, D, 1) || scn % 8 != 0)
+    return set_error(QFA_EINVAL, "quant: codes strides must be positive multiples of 16 bytes, token stride >= D");
+  return launch_quant(x, x_dtype, codes, scale_f32, scale_lp, scale_lp_dtype, zp, rowsum, B, H, N, D, sxb, sxh, sxn,
+                      scb, sch, scn, (hipStream_t)stream);
+}
+
+int qfa_dequant_per_token(const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp, void *out,
+                          int out_dtype, int64_t B, int64_t H, int64_t N, int D, int64_t scb, int64_t sch,
+                          int64_t scn, int64_t sob, int64_t soh, int64_t son, void *stream) {
+  if (!codes || !scale || !zp || !out) return set_error(QFA_EINVAL, "dequant: null pointer");
+  if (!is_float_dtype(scale_dtype) || !is_float_dtype(out_dtype))
+    return set_error(QFA_EINVAL, "dequant: bad scale_dtype/out_dtype");
+  if (B <= 0 || H <= 0 || N <= 0) return set_error(QFA_EINVAL, "dequant: B, H, N must be positive");
+  if (D != 32 && D != 64 && D != 128 && D != 256)
+    return set_error(QFA_EUNSUPPORTED, "dequant: head_dim %d not in {32, 64, 128, 256}", D);
+  if (!aligned16(codes) || !aligned16(out)) return set_error(QFA_EINVAL, "dequant: codes and out must be 16-byte aligned");
+  if (!strides_ok(scb, sch, scn, D, 1) || !strides_ok(sob, soh, son, D, elem_size(out_dtype)))
+    return set_error(QFA_EINVAL, "dequant: strides must be positive multiples of 16 bytes, token stride >= D");
+  return launch_dequant(codes, scale, scale_dtype, zp, out, out_dtype, B, H, N, D, scb, sch, scn, sob, soh, son,
+                        (hipStream_t)stream);
+}
+
+static int check_attn_common(const char *who, const AttnArgs &a) {
+  if (!a.qc || !a.sq || !a.zq || !a.rq || !a.kc || !a.sk || !a.zk || !a.rk || !a.v || !a.o || !a.lse)
+    return set_error(QFA_EINVAL, "%s: null pointer argument", who);
+  if (a.io_dtype != QFA_BF16 && a.io_dtype != QFA_F16)
+    return set_error(QFA_EINVAL, "%s: io_dtype must be QFA_BF16 or QFA_F16", who);
+  if (a.B <= 0 || a.H <= 0 || a.Nq <= 0 || a.Nk <= 0) return set_error(QFA_EINVAL, "%s: B, H, Nq, Nk must be positive", who);
+  if (a.Nq > 0x7fffff00LL || a.Nk > 0x7fffff00LL) return set_error(QFA_EUNSUPPORTED, "%s: sequence too long", who);
+  if (a.D != 64 && a.D != 128) return set_error(QFA_EUNSUPPORTED, "%s: head_dim %d not in {64, 128}", who, a.D);
+  if (!(a.sm_scale > 0.0f) || !(a.sm_scale < 3.0e38f))
+    return set_error(QFA_EINVAL, "%s: sm_scale must be a positive finite number", who);
+  if (a.causal && a.Nq != a.Nk) return set_error(QFA_EUNSUPPORTED, "%s: causal needs Nq == Nk", who);
+  if (!aligned16(a.qc) || !aligned16(a.kc) || !aligned16(a.v) || !aligned16(a.o))
+    return set_error(QFA_EINVAL, "%s: qc, kc, v, o must be 16-byte aligned", who);
+  if (!strides_ok(a.sqb, a.sqh, a.sqn, a.D, 1) || !strides_ok(a.skb, a.skh, a.skn, a.D, 1) ||
+      !strides_ok(a.svb, a.svh, a.svn, a.D, 2) || !strides_ok(a.sob, a.soh, a.son, a.D, 2))
+    return set_error(QFA_EINVAL, "%s: strides must be positive multiples of 16 bytes, token stride >= D", who);
+  return 0;
+}
+
+int qfa_attn_fwd(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,
+                 const float *sk, const int8_t *zk, const int32_t *rk, const void *v, void *o, float *lse,
+                 int io_dtype, int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D, int64_t sqb, int64_t sqh,
+                 int64_t sqn, int64_t skb, int64_t skh, int64_t skn, int64_t svb, int64_t svh, int64_t svn,
+                 int64_t sob, int64_t soh, int64_t son, float sm_scale, int causal, void *stream) {
+  AttnArgs a;
+  memset(&a, 0, sizeof(a));
+  a.qc = qc; a.sq = sq; a.zq = zq; a.rq = rq; a.kc = kc; a.sk = sk; a.zk = zk; a.rk = rk;
+  a.v = v; a.o = o; a.lse = lse; a.io_dtype = io_dtype;
+  a.B = B; a.H = H; a.Nq = Nq; a.Nk = Nk; a.D = D;
+  a.sqb = sqb; a.sqh = sqh; a.sqn = sqn; a.skb = skb; a.skh = skh; a.skn = skn;
+  a.svb = svb; a.svh = svh; a.svn = svn; a.sob = sob; a.soh = soh; a.son = son;
+  a.sm_scale = sm_scale; a.causal = causal;
+  if (int e = check_attn_common("attn_fwd", a)) return e;
+  return launch_fwd(a, (hipStream_t)stream);
+}
+
+int qfa_bwd_delta(const void *o, const void *dout, float *delta, int io_dtype, int64_t B, int64_t H, int64_t N,
+                  int D, int64_t sob, int64_t soh, int64_t son, int64_t sdb, int64_t sdh, int64_t sdn,
+                  void *stream) {
+  if (!o || !dout || !delta) return set_error(QFA_EINVAL, "bwd_delta: null pointer argument");
+  if (io_dtype != QFA_BF16 && io_dtype != QFA_F16) return set_error(QFA_EINVAL, "bwd_delta: io_dtype must be QFA_BF16 or QFA_F16");
+  if (B <= 0 || H <= 0 || N <= 0) return set_error(QFA_EINVAL, "bwd_delta: B, H, N must be positive");
+  if (D != 64 && D != 128) return set_error(QFA_EUNSUPPORTED, "bwd_delta: head_dim %d not in {64, 128}", D);
+  if (!aligned16(o) || !aligned16(dout)) return set_error(QFA_EINVAL, "bwd_delta: o and dout must be 16-byte aligned");
+  if (!strides_ok(sob, soh, son, D, 2) || !strides_ok(sdb, sdh, sdn, D, 2))
+    return set_error(QFA_EINVAL, "bwd_delta: strides must be positive multiples of 16 bytes, token stride >= D");
+  return launch_delta(o, dout, delta, io_dtype, B, H, N, D, sob, soh, son, sdb, sdh, sdn, (hipStream_t)stream);
+}
+
+int qfa_attn_bwd(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,
+                 const float *sk, const int8_t *zk, const int32_t *rk, const void *v, const void *o,
+                 const void *dout, const float *lse, float *delta, void *dq, void *dk, void *dv, int io_dtype,
+                 int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D, int64_t sqb, int64_t sqh, int64_t sqn,
+                 int64_t skb, int64_t skh, int64_t skn, int64_t svb, int64_t svh, int64_t svn, int64_t sob,
+                 int64_t soh, int64_t son, int64_t sdob, int64_t sdoh, int64_t sdon, int64_t sdqb, int64_t sdqh,
+                 int64_t sdqn, int64_t sdkb, int64_t sdkh, int64_t sdkn, int64_t sdvb, int64_t sdvh,
+                 int64_t sdvn, float sm_scale, int causal, void *stream) {
+  AttnArgs a;
+  memset(&a, 0, sizeof(a));
+  a.qc = qc; a.sq = sq; a.zq = zq; a.rq = rq; a.kc = kc; a.sk = sk; a.zk = zk; a.rk = rk;
+  a.v = v; a.o = const_cast<void *>(o); a.lse = const_cast<float *>(lse); a.io_dtype = io_dtype;
+  a.dout = dout; a.delta = delta; a.dq = dq; a.dk = dk; a.dv = dv;
+  a.B = B; a.H = H; a.Nq = Nq; a.Nk = Nk; a.D = D;
+  a.sqb = sqb; a.sqh = sqh; a.sqn = sqn; a.skb = skb; a.skh = skh; a.skn = skn;
+  a.svb = svb; a.svh = svh; a.svn = svn; a.sob = sob; a.soh = soh; a.son = son;
+  a.sdob = sdob; a.sdoh = sdoh; a.sdon = sdon; a.sdqb = sdqb; a.sdqh = sdqh; a.sdqn = sdqn;
+  a.sdkb = sdkb; a.sdkh = sdkh; a.sdkn = sdkn; a.sdvb = sdvb; a.sdvh = sdvh; a.sdvn = sdvn;
+  a.sm_scale = sm_scale; a.causal = causal;
+  if (int e = check_attn_common("attn_bwd", a)) return e;
+  if (!dout || !delta || !dq || !dk || !dv) return set_error(QFA_EINVAL, "attn_bwd: null pointer argument");
+  if (!aligned16(dout) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv))
+    return set_error(QFA_EINVAL, "attn_bwd: dout, dq, dk, dv must be 16-byte aligned");
+  if (!strides_ok(sdob, sdoh, sdon, D, 2) || !strides_ok(sdqb, sdqh, sdqn, D, 2) ||
+      !strides_ok(sdkb, sdkh, sdkn, D, 2) || !strides_ok(sdvb, sdvh, sdvn, D, 2))
+    return set_error(QFA_EINVAL, "attn_bwd: strides must be positive multiples of 16 bytes, token stride >= D");
+  if (int e = launch_delta(o, dout, delta, io_dtype, B, H, Nq, D, sob, soh, son, sdob, sdoh, sdon, (hipStream_t)stream))
+    return e;
+  return launch_bwd(a, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,84 @@
+// Device-side helpers shared by the gfx950 kernels: vector types, MFMA wrappers,
+// DPP lane exchanges, 16-bit float conversions.  gfx950 (CDNA4) only, wave64.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace qfa {
+
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// ---- 16-bit float element traits ------------------------------------------------------------
+template <typename T> struct Elem;
+template <> struct Elem<__bf16> {
+  typedef bf16x2 x2;
+  typedef bf16x4 x4;
+  typedef bf16x8 x8;
+};
+template <> struct Elem<_Float16> {
+  typedef f16x2 x2;
+  typedef f16x4 x4;
+  typedef f16x8 x8;
+};
+
+// two fp32 -> packed pair of 16-bit floats (round to nearest even), as one dword
+template <typename T> __device__ __forceinline__ unsigned pack2(float a, float b) {
+  f32x2 p = {a, b};
+  typename Elem<T>::x2 q = __builtin_convertvector(p, typename Elem<T>::x2);
+  return __builtin_bit_cast(unsigned, q);
+}
+template <typename T> __device__ __forceinline__ float lo_to_f32(unsigned w) {
+  typename Elem<T>::x2 q = __builtin_bit_cast(typename Elem<T>::x2, w);
+  return (float)q[0];
+}
+template <typename T> __device__ __forceinline__ float hi_to_f32(unsigned w) {
+  typename Elem<T>::x2 q = __builtin_bit_cast(typename Elem<T>::x2, w);
+  return (float)q[1];
+}
+
+// ---- MFMA wrappers (A and B: 16 bytes per lane; C/D: 16 dwords per lane) ------------------------
+// 32x32x32 int8:  A lane l = row l%32, 16 consecutive k at k-group l/32;  B lane l = column l%32,
+// same k slots;  D lane l = column l%32, register v = row 8*(v/4) + 4*(l/32) + v%4.
+__device__ __forceinline__ i32x16 mfma_i8(i32x4 a, i32x4 b, i32x16 c) {
+  return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+}
+// 32x32x16 bf16/f16: A lane l = row l%32, 8 consecutive k at k-group l/32; B likewise; D as above.
+template <typename T> __device__ __forceinline__ f32x16 mfma_16b(u32x4 a, u32x4 b, f32x16 c);
+template <> __device__ __forceinline__ f32x16 mfma_16b<__bf16>(u32x4 a, u32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
+                                                 0, 0);
+}
+template <> __device__ __forceinline__ f32x16 mfma_16b<_Float16>(u32x4 a, u32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
+                                                0);
+}
+
+// ---- lane exchanges ---------------------------------------------------------------------------
+// DPP controls: quad_perm [1,0,3,2] = 0xB1, [2,3,0,1] = 0x4E, row_half_mirror = 0x141, row_mirror = 0x140
+template <int CTRL> __device__ __forceinline__ float dpp_f(float x) {
+  int xi = __builtin_bit_cast(int, x);
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(xi, xi, CTRL, 0xf, 0xf, false));
+}
+template <int CTRL> __device__ __forceinline__ int dpp_i(int x) {
+  return __builtin_amdgcn_update_dpp(x, x, CTRL, 0xf, 0xf, false);
+}
+// value held by lane (l ^ 32)
+__device__ __forceinline__ float swap32_f(float x) { return __shfl_xor(x, 32, 64); }
+
+}  // namespace qfa

@@ -1,0 +1,43 @@
+// Host-side declarations shared by the translation units of libqfa.so: the error
+// channel behind qfa_last_error() and the launchers the C entry points dispatch to.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/qfa.h"
+
+namespace qfa {
+
+// Records a thread-local message and returns `code` (so `return set_error(...)` reads naturally).
+int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+// hipGetLastError() after a launch; 0 or the positive hipError_t, with the message recorded.
+int check_launch(const char *what);
+
+int launch_quant(const void *x, int x_dtype, int8_t *codes, float *scale, void *scale_lp, int scale_lp_dtype,
+                 int8_t *zp, int32_t *rowsum, int64_t B, int64_t H, int64_t N, int D, int64_t sxb, int64_t sxh,
+                 int64_t sxn, int64_t scb, int64_t sch, int64_t scn, hipStream_t st);
+int launch_dequant(const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp, void *out,
+                   int out_dtype, int64_t B, int64_t H, int64_t N, int D, int64_t scb, int64_t sch, int64_t scn,
+                   int64_t sob, int64_t soh, int64_t son, hipStream_t st);
+
+// Tensors of one attention call, after validation.  Strides in elements.
+struct AttnArgs {
+  const int8_t *qc; const float *sq; const int8_t *zq; const int32_t *rq;
+  const int8_t *kc; const float *sk; const int8_t *zk; const int32_t *rk;
+  const void *v; void *o; float *lse;
+  const void *dout; float *delta; void *dq; void *dk; void *dv;   // backward only
+  int64_t B, H, Nq, Nk;
+  int64_t sqb, sqh, sqn, skb, skh, skn, svb, svh, svn, sob, soh, son;
+  int64_t sdob, sdoh, sdon, sdqb, sdqh, sdqn, sdkb, sdkh, sdkn, sdvb, sdvh, sdvn;
+  float sm_scale;
+  int causal;
+  int D;
+  int io_dtype;
+};
+
+int launch_fwd(const AttnArgs &a, hipStream_t st);
+int launch_delta(const void *o, const void *dout, float *delta, int io_dtype, int64_t B, int64_t H, int64_t N, int D,
+                 int64_t sob, int64_t soh, int64_t son, int64_t sdb, int64_t sdh, int64_t sdn, hipStream_t st);
+int launch_bwd(const AttnArgs &a, hipStream_t st);
+
+}  // namespace qfa

@@ -1,0 +1,264 @@
+// Per-token asymmetric INT8 quantizer and its inverse for gfx950.
+//
+// Arithmetic contract (asymmetric_quant.py:66-106 of the reference): per token row,
+//   scale = (max - min) / 255 (1 if 0);  zp = clamp(roundf(-128 - min/scale));
+//   code  = clamp(roundf(x/scale + zp)),  every step one IEEE binary32 operation.
+// This file is compiled with -ffp-contract=off and without fast-math so that `/` is the
+// correctly rounded division and nothing is fused or re-associated: codes and zero points
+// are bit-identical to a CPU evaluation of the same expressions.
+//
+// Mapping: a token of D elements is held by D/8 adjacent lanes (8 elements = one 16-byte
+// load per lane for 16-bit inputs, two for fp32), so one wave64 load instruction covers
+// 512/D tokens with fully coalesced 16-byte accesses.  The row is read once, kept in
+// registers, reduced with DPP lane permutes inside the lane group (no LDS), and the codes
+// leave as one 8-byte store per lane.  HBM-bound: D*sizeof(in) + D + 9 bytes per token
+// (+2 with the 16-bit scale copy).
+#include "qfa_device.h"
+#include "qfa_host.h"
+
+namespace qfa {
+
+template <int LPT> __device__ __forceinline__ float group_min(float v) {
+  v = fminf(v, dpp_f<0xB1>(v));
+  if (LPT >= 4) v = fminf(v, dpp_f<0x4E>(v));
+  if (LPT >= 8) v = fminf(v, dpp_f<0x141>(v));
+  if (LPT >= 16) v = fminf(v, dpp_f<0x140>(v));
+  if (LPT >= 32) v = fminf(v, __shfl_xor(v, 16, 64));
+  return v;
+}
+template <int LPT> __device__ __forceinline__ float group_max(float v) {
+  v = fmaxf(v, dpp_f<0xB1>(v));
+  if (LPT >= 4) v = fmaxf(v, dpp_f<0x4E>(v));
+  if (LPT >= 8) v = fmaxf(v, dpp_f<0x141>(v));
+  if (LPT >= 16) v = fmaxf(v, dpp_f<0x140>(v));
+  if (LPT >= 32) v = fmaxf(v, __shfl_xor(v, 16, 64));
+  return v;
+}
+template <int LPT> __device__ __forceinline__ int group_sum(int v) {
+  v += dpp_i<0xB1>(v);
+  if (LPT >= 4) v += dpp_i<0x4E>(v);
+  if (LPT >= 8) v += dpp_i<0x141>(v);
+  if (LPT >= 16) v += dpp_i<0x140>(v);
+  if (LPT >= 32) v += __shfl_xor(v, 16, 64);
+  return v;
+}
+
+template <typename T> struct Load8;
+template <> struct Load8<float> {
+  static __device__ __forceinline__ void run(const void *p, float (&v)[8]) {
+    const f32x4 *q = reinterpret_cast<const f32x4 *>(p);
+    f32x4 a = __builtin_nontemporal_load(q), b = __builtin_nontemporal_load(q + 1);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { v[e] = a[e]; v[4 + e] = b[e]; }
+  }
+};
+template <> struct Load8<__bf16> {
+  static __device__ __forceinline__ void run(const void *p, float (&v)[8]) {
+    u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {   // bf16 -> fp32 is a 16-bit shift
+      v[2 * e] = __builtin_bit_cast(float, w[e] << 16);
+      v[2 * e + 1] = __builtin_bit_cast(float, w[e] & 0xffff0000u);
+    }
+  }
+};
+template <> struct Load8<_Float16> {
+  static __device__ __forceinline__ void run(const void *p, float (&v)[8]) {
+    f16x8 w = __builtin_bit_cast(f16x8, __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p)));
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (float)w[e];
+  }
+};
+
+struct QuantArgs {
+  const void *x;
+  int8_t *codes;
+  float *scale;
+  void *scale_lp;
+  int8_t *zp;
+  int32_t *rowsum;
+  int64_t N;
+  int64_t H;
+  int64_t sxb, sxh, sxn, scb, sch, scn;
+  int chunks_per_bh;  // ceil(N / tokens per block)
+  int scale_lp_dtype;
+};
+
+// One block = 256 threads = U passes over 256/(D/8) tokens of one (b,h) slice.
+template <typename T, int D, int U> __global__ __launch_bounds__(256) void quant_kernel(QuantArgs a) {
+  constexpr int LPT = D / 8;          // lanes per token
+  constexpr int TPP = 256 / LPT;      // tokens per pass
+  const int tid = threadIdx.x;
+  const int sub = tid % LPT;
+  const int64_t bh = blockIdx.x / a.chunks_per_bh;
+  const int64_t chunk = blockIdx.x % a.chunks_per_bh;
+  const int64_t b = bh / a.H, h = bh % a.H;
+  const int64_t n0 = chunk * (int64_t)(TPP * U) + tid / LPT;
+  const T *xb = reinterpret_cast<const T *>(a.x) + b * a.sxb + h * a.sxh;
+  int8_t *cb = a.codes + b * a.scb + h * a.sch;
+
+  float v[U][8];
+  bool live[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t n = n0 + (int64_t)u * TPP;
+    live[u] = n < a.N;
+    const int64_t nn = live[u] ? n : a.N - 1;   // tail lanes re-read the last token, never store
+    Load8<T>::run(xb + nn * a.sxn + sub * 8, v[u]);
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t n = n0 + (int64_t)u * TPP;
+    float mn = v[u][0], mx = v[u][0];
+#pragma unroll
+    for (int e = 1; e < 8; ++e) { mn = fminf(mn, v[u][e]); mx = fmaxf(mx, v[u][e]); }
+    mn = group_min<LPT>(mn);
+    mx = group_max<LPT>(mx);
+    float scale = (mx - mn) / 255.0f;
+    scale = (scale == 0.0f) ? 1.0f : scale;
+    const float zpf = -128.0f - mn / scale;
+    const float zp = fmaxf(-128.0f, fminf(127.0f, __builtin_roundf(zpf)));
+    int c[8];
+    int sum = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float y = v[u][e] / scale + zp;
+      c[e] = (int)fmaxf(-128.0f, fminf(127.0f, __builtin_roundf(y)));
+      sum += c[e];
+    }
+    sum = group_sum<LPT>(sum);
+    if (live[u]) {
+      u32x2 w;
+      w[0] = (c[0] & 0xff) | ((c[1] & 0xff) << 8) | ((c[2] & 0xff) << 16) | ((unsigned)c[3] << 24);
+      w[1] = (c[4] & 0xff) | ((c[5] & 0xff) << 8) | ((c[6] & 0xff) << 16) | ((unsigned)c[7] << 24);
+      *reinterpret_cast<u32x2 *>(cb + n * a.scn + sub * 8) = w;
+      if (sub == 0) {
+        const int64_t t = bh * a.N + n;
+        a.scale[t] = scale;
+        a.zp[t] = (int8_t)(int)zp;
+        if (a.rowsum) a.rowsum[t] = sum;
+        if (a.scale_lp) {
+          if (a.scale_lp_dtype == QFA_F16) reinterpret_cast<_Float16 *>(a.scale_lp)[t] = (_Float16)scale;
+          else reinterpret_cast<__bf16 *>(a.scale_lp)[t] = (__bf16)scale;
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int D> static int launch_quant_d(const QuantArgs &a0, int64_t BH, hipStream_t st) {
+  constexpr int U = 4;
+  constexpr int TOK = (256 / (D / 8)) * U;
+  QuantArgs a = a0;
+  const int64_t chunks = (a.N + TOK - 1) / TOK;
+  if (chunks * BH > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "quant: too many tokens for one launch");
+  a.chunks_per_bh = (int)chunks;
+  quant_kernel<T, D, U><<<dim3((unsigned)(chunks * BH)), dim3(256), 0, st>>>(a);
+  return check_launch("qfa_quant_per_token");
+}
+template <typename T> static int launch_quant_t(const QuantArgs &a, int D, int64_t BH, hipStream_t st) {
+  switch (D) {
+    case 32: return launch_quant_d<T, 32>(a, BH, st);
+    case 64: return launch_quant_d<T, 64>(a, BH, st);
+    case 128: return launch_quant_d<T, 128>(a, BH, st);
+    case 256: return launch_quant_d<T, 256>(a, BH, st);
+  }
+  return set_error(QFA_EUNSUPPORTED, "quant: head_dim must be 32, 64, 128 or 256");
+}
+
+int launch_quant(const void *x, int x_dtype, int8_t *codes, float *scale, void *scale_lp, int scale_lp_dtype,
+                 int8_t *zp, int32_t *rowsum, int64_t B, int64_t H, int64_t N, int D, int64_t sxb, int64_t sxh,
+                 int64_t sxn, int64_t scb, int64_t sch, int64_t scn, hipStream_t st) {
+  QuantArgs a;
+  a.x = x; a.codes = codes; a.scale = scale; a.scale_lp = scale_lp; a.zp = zp; a.rowsum = rowsum;
+  a.N = N; a.H = H; a.sxb = sxb; a.sxh = sxh; a.sxn = sxn; a.scb = scb; a.sch = sch; a.scn = scn;
+  a.chunks_per_bh = 0; a.scale_lp_dtype = scale_lp_dtype;
+  switch (x_dtype) {
+    case QFA_F32: return launch_quant_t<float>(a, D, B * H, st);
+    case QFA_F16: return launch_quant_t<_Float16>(a, D, B * H, st);
+    case QFA_BF16: return launch_quant_t<__bf16>(a, D, B * H, st);
+  }
+  return set_error(QFA_EINVAL, "quant: bad x_dtype");
+}
+
+// ---------------------------------------------------------------------------------------------
+// Dequantize: out = (code - zp) * scale  (asymmetric_quant.py:160), 8 elements per lane.
+struct DequantArgs {
+  const int8_t *codes;
+  const void *scale;
+  const int8_t *zp;
+  void *out;
+  int64_t N, H;
+  int64_t scb, sch, scn, sob, soh, son;
+  int chunks_per_bh;
+  int scale_dtype;
+};
+
+template <typename TO, int D> __global__ __launch_bounds__(256) void dequant_kernel(DequantArgs a) {
+  constexpr int LPT = D / 8;
+  constexpr int TPP = 256 / LPT;
+  const int tid = threadIdx.x;
+  const int sub = tid % LPT;
+  const int64_t bh = blockIdx.x / a.chunks_per_bh;
+  const int64_t chunk = blockIdx.x % a.chunks_per_bh;
+  const int64_t b = bh / a.H, h = bh % a.H;
+  const int64_t n = chunk * (int64_t)TPP + tid / LPT;
+  if (n >= a.N) return;
+  const int64_t t = bh * a.N + n;
+  float scale;
+  if (a.scale_dtype == QFA_F32) scale = reinterpret_cast<const float *>(a.scale)[t];
+  else if (a.scale_dtype == QFA_F16) scale = (float)reinterpret_cast<const _Float16 *>(a.scale)[t];
+  else scale = (float)reinterpret_cast<const __bf16 *>(a.scale)[t];
+  const float zp = (float)a.zp[t];
+  const u32x2 w = *reinterpret_cast<const u32x2 *>(a.codes + b * a.scb + h * a.sch + n * a.scn + sub * 8);
+  float f[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int c = (int)(int8_t)((w[e / 4] >> (8 * (e % 4))) & 0xff);
+    f[e] = ((float)c - zp) * scale;
+  }
+  TO *o = reinterpret_cast<TO *>(a.out) + b * a.sob + h * a.soh + n * a.son + sub * 8;
+  if constexpr (sizeof(TO) == 4) {
+    f32x4 lo = {f[0], f[1], f[2], f[3]}, hi = {f[4], f[5], f[6], f[7]};
+    reinterpret_cast<f32x4 *>(o)[0] = lo;
+    reinterpret_cast<f32x4 *>(o)[1] = hi;
+  } else {
+    u32x4 p;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) p[e] = pack2<TO>(f[2 * e], f[2 * e + 1]);
+    *reinterpret_cast<u32x4 *>(o) = p;
+  }
+}
+
+template <typename TO> static int launch_dequant_t(DequantArgs a, int D, int64_t BH, hipStream_t st) {
+  const int tpp = 256 / (D / 8);
+  const int64_t chunks = (a.N + tpp - 1) / tpp;
+  if (chunks * BH > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "dequant: too many tokens for one launch");
+  a.chunks_per_bh = (int)chunks;
+  const dim3 grid((unsigned)(chunks * BH)), block(256);
+  switch (D) {
+    case 32: dequant_kernel<TO, 32><<<grid, block, 0, st>>>(a); break;
+    case 64: dequant_kernel<TO, 64><<<grid, block, 0, st>>>(a); break;
+    case 128: dequant_kernel<TO, 128><<<grid, block, 0, st>>>(a); break;
+    case 256: dequant_kernel<TO, 256><<<grid, block, 0, st>>>(a); break;
+    default: return set_error(QFA_EUNSUPPORTED, "dequant: head_dim must be 32, 64, 128 or 256");
+  }
+  return check_launch("qfa_dequant_per_token");
+}
+
+int launch_dequant(const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp, void *out,
+                   int out_dtype, int64_t B, int64_t H, int64_t N, int D, int64_t scb, int64_t sch, int64_t scn,
+                   int64_t sob, int64_t soh, int64_t son, hipStream_t st) {
+  DequantArgs a;
+  a.codes = codes; a.scale = scale; a.zp = zp; a.out = out; a.N = N; a.H = H;
+  a.scb = scb; a.sch = sch; a.scn = scn; a.sob = sob; a.soh = soh; a.son = son;
+  a.chunks_per_bh = 0; a.scale_dtype = scale_dtype;
+  switch (out_dtype) {
+    case QFA_F32: return launch_dequant_t<float>(a, D, B * H, st);
+    case QFA_F16: return launch_dequant_t<_Float16>(a, D, B * H, st);
+    case QFA_BF16: return launch_dequant_t<__bf16>(a, D, B * H, st);
+  }
+  return set_error(QFA_EINVAL, "dequant: bad out_dtype");
+}
+
+}  // namespace qfa

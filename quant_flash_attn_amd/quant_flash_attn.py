@@ -1,0 +1,191 @@
+"""INT8 per-token quantized flash attention -- drop-in for the reference's quant_flash_attn.py.
+
+Two autograd entry points, both backed by the HIP kernels behind qfa_attn_fwd / qfa_attn_bwd:
+
+  QuantFlashAttnQKV.apply(q, k, v, causal, sm_scale)            (alias quant_flash_attn_qkv)
+      Signature of the repository's fused-attention Function (flash_attn_triton.py:441).  Q and K
+      are quantized per token inside (asymmetric_quant.py math), QK^T runs on INT8 MFMA, V stays
+      in 16-bit.  Gradients flow straight through the quantizer to q and k.
+
+  QuantFlashAttention.apply(q, kv_fp16, kv_quant, sm_scale)     (alias quant_flash_attn)
+      The reference's own entry point (quant_flash_attn.py:173-240): one quantized tensor serves as
+      K and V, `kv_fp16` only receives the gradient, backward returns (dq, dkv, None, None) with
+      dkv = dK + dV (:161).  Difference from the reference, stated: Q is quantized per token too
+      (the reference keeps Q in fp16), because the score product runs on INT8 MFMA.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from .asymmetric_quant import QuantizedTokens, dequantize_per_token, quantize_for_attention
+
+_IO_DTYPES = (torch.bfloat16, torch.float16)
+
+
+def _flat(t: torch.Tensor, dtype: torch.dtype, n: int, name: str) -> torch.Tensor:
+    t = t.reshape(-1)
+    if t.dtype != dtype or t.numel() != n:
+        raise ValueError(f"{name}: expected {n} values of {dtype}, got {t.numel()} of {t.dtype}")
+    return t.contiguous()
+
+
+def _rows16(t: torch.Tensor) -> torch.Tensor:
+    """[B,H,N,D] tensor whose rows are contiguous and whose strides / base are 16-byte multiples."""
+    es = t.element_size()
+    ok = (t.stride(3) == 1 and t.stride(2) >= t.shape[3] and t.data_ptr() % 16 == 0
+          and all(t.stride(i) > 0 and (t.stride(i) * es) % 16 == 0 for i in range(3)))
+    return t if ok else t.contiguous()
+
+
+def _unpack(qt: QuantizedTokens, name: str):
+    codes, scale, zp, rowsum = qt
+    if codes.dim() != 4 or codes.dtype != torch.int8:
+        raise ValueError(f"{name}.codes must be a 4-D int8 tensor")
+    n = codes.shape[0] * codes.shape[1] * codes.shape[2]
+    return (_rows16(codes), _flat(scale, torch.float32, n, f"{name}.scale"),
+            _flat(zp, torch.int8, n, f"{name}.zero_point"), _flat(rowsum, torch.int32, n, f"{name}.rowsum"))
+
+
+def attn_fwd_quantized(qq: QuantizedTokens, kq: QuantizedTokens, v: torch.Tensor, causal: bool,
+                       sm_scale: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """O, LSE = attention(dequant(qq), dequant(kq), v).  v and O are bf16 or fp16 [B,H,N,D];
+    LSE is fp32 [B,H,Nq] (natural log, as quant_flash_attn.py:79)."""
+    if v.dtype not in _IO_DTYPES:
+        raise TypeError(f"v must be bfloat16 or float16, got {v.dtype}")
+    qc, sq, zq, rq = _unpack(qq, "q")
+    kc, sk, zk, rk = _unpack(kq, "k")
+    _lib.require_gpu(qc, sq, zq, rq, kc, sk, zk, rk, v)
+    B, H, Nq, D = qc.shape
+    Nk = kc.shape[2]
+    if kc.shape != (B, H, Nk, D) or v.shape != (B, H, Nk, D):
+        raise ValueError(f"shape mismatch: q {tuple(qc.shape)}, k {tuple(kc.shape)}, v {tuple(v.shape)}")
+    v = _rows16(v)
+    o = torch.empty((B, H, Nq, D), dtype=v.dtype, device=v.device)
+    lse = torch.empty((B, H, Nq), dtype=torch.float32, device=v.device)
+    with torch.cuda.device(v.device):
+        code = _lib.lib().qfa_attn_fwd(
+            qc.data_ptr(), sq.data_ptr(), zq.data_ptr(), rq.data_ptr(),
+            kc.data_ptr(), sk.data_ptr(), zk.data_ptr(), rk.data_ptr(),
+            v.data_ptr(), o.data_ptr(), lse.data_ptr(), _lib.DTYPE_CODE[v.dtype],
+            B, H, Nq, Nk, D,
+            qc.stride(0), qc.stride(1), qc.stride(2), kc.stride(0), kc.stride(1), kc.stride(2),
+            v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1), o.stride(2),
+            float(sm_scale), int(bool(causal)), _lib.stream_of(v))
+    _lib.check(code, "qfa_attn_fwd")
+    return o, lse
+
+
+def attn_bwd_quantized(qq: QuantizedTokens, kq: QuantizedTokens, v: torch.Tensor, o: torch.Tensor,
+                       do: torch.Tensor, lse: torch.Tensor, causal: bool, sm_scale: float
+                       ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """dQ, dK, dV (w.r.t. the dequantized q^, k^ and v) in v's dtype."""
+    if v.dtype not in _IO_DTYPES:
+        raise TypeError(f"v must be bfloat16 or float16, got {v.dtype}")
+    qc, sq, zq, rq = _unpack(qq, "q")
+    kc, sk, zk, rk = _unpack(kq, "k")
+    B, H, Nq, D = qc.shape
+    Nk = kc.shape[2]
+    if o.shape != (B, H, Nq, D) or do.shape != (B, H, Nq, D) or v.shape != (B, H, Nk, D):
+        raise ValueError("shape mismatch between o / do / v and the quantized tensors")
+    if o.dtype != v.dtype:
+        raise TypeError("o and v must have the same dtype")
+    if do.dtype != v.dtype:
+        do = do.to(v.dtype)
+    _lib.require_gpu(qc, kc, v, o, do, lse)
+    v, o, do = _rows16(v), _rows16(o), _rows16(do)
+    lse = _flat(lse, torch.float32, B * H * Nq, "lse")
+    delta = torch.empty((B, H, Nq), dtype=torch.float32, device=v.device)
+    dq = torch.empty((B, H, Nq, D), dtype=v.dtype, device=v.device)
+    dk = torch.empty((B, H, Nk, D), dtype=v.dtype, device=v.device)
+    dv = torch.empty((B, H, Nk, D), dtype=v.dtype, device=v.device)
+    s = lambda t: (t.stride(0), t.stride(1), t.stride(2))
+    with torch.cuda.device(v.device):
+        code = _lib.lib().qfa_attn_bwd(
+            qc.data_ptr(), sq.data_ptr(), zq.data_ptr(), rq.data_ptr(),
+            kc.data_ptr(), sk.data_ptr(), zk.data_ptr(), rk.data_ptr(),
+            v.data_ptr(), o.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), _lib.DTYPE_CODE[v.dtype],
+            B, H, Nq, Nk, D, *s(qc), *s(kc), *s(v), *s(o), *s(do), *s(dq), *s(dk), *s(dv),
+            float(sm_scale), int(bool(causal)), _lib.stream_of(v))
+    _lib.check(code, "qfa_attn_bwd")
+    return dq, dk, dv
+
+
+def _io_dtype(t: torch.Tensor) -> torch.dtype:
+    return t.dtype if t.dtype in _IO_DTYPES else torch.bfloat16
+
+
+class QuantFlashAttnQKV(torch.autograd.Function):
+    """forward(ctx, q, k, v, causal, sm_scale) -> o   (argument order of flash_attn_triton.py:441).
+
+    q, k, v: [B,H,N,D] bf16 / fp16 (fp32 is accepted: V and O then pass through bf16).
+    causal keeps key j for query i when j <= i (flash_attn_triton.py:50)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, causal, sm_scale):
+        _lib.require_gpu(q, k, v)
+        if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+            raise ValueError("q, k, v must be 4-D (Batch, Heads, Seq, Head_Dim)")
+        if q.shape[-1] != k.shape[-1] or k.shape != v.shape or q.shape[:2] != k.shape[:2]:
+            raise ValueError(f"shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
+        qq = quantize_for_attention(q)
+        kq = quantize_for_attention(k)
+        v16 = v.to(_io_dtype(v))
+        o, lse = attn_fwd_quantized(qq, kq, v16, causal, sm_scale)
+        ctx.save_for_backward(*qq, *kq, v16, o, lse)
+        ctx.causal, ctx.sm_scale = bool(causal), float(sm_scale)
+        ctx.in_dtypes = (q.dtype, k.dtype, v.dtype)
+        return o.to(q.dtype)
+
+    @staticmethod
+    def backward(ctx, do):
+        t = ctx.saved_tensors
+        qq, kq = QuantizedTokens(*t[0:4]), QuantizedTokens(*t[4:8])
+        v16, o, lse = t[8], t[9], t[10]
+        dq, dk, dv = attn_bwd_quantized(qq, kq, v16, o, do.to(v16.dtype), lse, ctx.causal, ctx.sm_scale)
+        dq_t, dk_t, dv_t = ctx.in_dtypes
+        return dq.to(dq_t), dk.to(dk_t), dv.to(dv_t), None, None
+
+
+quant_flash_attn_qkv = QuantFlashAttnQKV.apply
+
+
+class QuantFlashAttention(torch.autograd.Function):
+    """forward(ctx, q, kv_fp16, kv_quant, sm_scale) -> o; backward -> (dq, dkv, None, None).
+
+    Positional contract of the reference (quant_flash_attn.py:178-237): kv_quant is the
+    (codes, scale, zero_point) tuple returned by asymmetric_quant_per_token, kv_fp16 is only a
+    placeholder leaf that receives dkv, attention is non-causal, K == V == dequant(kv_quant)."""
+
+    @staticmethod
+    def forward(ctx, q, kv_fp16, kv_quant, sm_scale):
+        codes, scale, zp = kv_quant
+        _lib.require_gpu(q, codes, scale, zp)
+        if q.dim() != 4 or codes.shape != kv_fp16.shape or q.shape[-1] != codes.shape[-1]:
+            raise ValueError(f"shape mismatch: q {tuple(q.shape)}, kv {tuple(kv_fp16.shape)}, codes {tuple(codes.shape)}")
+        io = _io_dtype(q)
+        qq = quantize_for_attention(q)
+        # K operand: the caller's codes with the scale exactly as stored (fp16 in the reference)
+        kq = QuantizedTokens(codes, scale.to(torch.float32), zp,
+                             codes.sum(dim=-1, keepdim=True, dtype=torch.int32))
+        v16 = dequantize_per_token(codes, scale, zp, io)          # V operand: dequant(kv) (:65)
+        o, lse = attn_fwd_quantized(qq, kq, v16, False, sm_scale)
+        ctx.save_for_backward(*qq, *kq, v16, o, lse)
+        ctx.sm_scale = float(sm_scale)
+        ctx.q_dtype, ctx.kv_dtype = q.dtype, kv_fp16.dtype
+        return o.to(q.dtype)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        t = ctx.saved_tensors
+        qq, kq = QuantizedTokens(*t[0:4]), QuantizedTokens(*t[4:8])
+        v16, o, lse = t[8], t[9], t[10]
+        dq, dk, dv = attn_bwd_quantized(qq, kq, v16, o, grad_output.to(v16.dtype), lse, False, ctx.sm_scale)
+        dkv = dk.to(torch.float32).add_(dv).to(ctx.kv_dtype)      # :161 (dk already carries sm_scale)
+        return dq.to(ctx.q_dtype), dkv, None, None
+
+
+quant_flash_attn = QuantFlashAttention.apply

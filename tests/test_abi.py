@@ -1,0 +1,84 @@
+"""The C-ABI library: loads without a GPU, exports every symbol include/qfa.h declares, and
+rejects malformed calls with an error code and message before touching the device."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "qfa.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(qfa_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(qfa):
+    from quant_flash_attn_amd import _lib
+    names = _declared_symbols()
+    assert names == sorted(_lib._SIGNATURES), "python binding and include/qfa.h list different entry points"
+    handle = ctypes.CDLL(_lib.library_path())
+    for n in names:
+        assert hasattr(handle, n), f"libqfa.so does not export {n}"
+    assert _lib.lib().qfa_version() == 100
+
+
+def test_argument_errors_need_no_gpu(qfa):
+    from quant_flash_attn_amd import _lib
+    L = _lib.lib()
+    ok_ptr = 0x1000  # never dereferenced: validation fails first
+    # null pointer
+    rc = L.qfa_quant_per_token(None, 2, ok_ptr, ok_ptr, None, 0, ok_ptr, None, 1, 1, 8, 64, 512, 512, 64, 512, 512, 64, None)
+    assert rc == -1 and b"null" in L.qfa_last_error()
+    # bad dtype
+    rc = L.qfa_quant_per_token(ok_ptr, 7, ok_ptr, ok_ptr, None, 0, ok_ptr, None, 1, 1, 8, 64, 512, 512, 64, 512, 512, 64, None)
+    assert rc == -1 and b"x_dtype" in L.qfa_last_error()
+    # unsupported head_dim
+    rc = L.qfa_quant_per_token(ok_ptr, 2, ok_ptr, ok_ptr, None, 0, ok_ptr, None, 1, 1, 8, 48, 384, 384, 48, 384, 384, 48, None)
+    assert rc == -2 and b"head_dim" in L.qfa_last_error()
+    # misaligned pointer, bad stride
+    rc = L.qfa_quant_per_token(ok_ptr + 2, 2, ok_ptr, ok_ptr, None, 0, ok_ptr, None, 1, 1, 8, 64, 512, 512, 64, 512, 512, 64, None)
+    assert rc == -1 and b"aligned" in L.qfa_last_error()
+    rc = L.qfa_quant_per_token(ok_ptr, 2, ok_ptr, ok_ptr, None, 0, ok_ptr, None, 1, 1, 8, 64, 512, 512, 60, 512, 512, 64, None)
+    assert rc == -1 and b"strides" in L.qfa_last_error()
+    # attention: causal with Nq != Nk, bad sm_scale, bad head_dim
+    def fwd(Nq=128, Nk=128, D=64, sm=0.125, causal=0, io=2):
+        s = (Nq * D * 2, Nq * D, D)
+        return L.qfa_attn_fwd(*([ok_ptr] * 11), io, 1, 2, Nq, Nk, D, *s, *s, *s, *s, sm, causal, None)
+    assert fwd(Nq=64, Nk=128, causal=1) == -2 and b"causal" in L.qfa_last_error()
+    assert fwd(sm=0.0) == -1 and b"sm_scale" in L.qfa_last_error()
+    assert fwd(D=96) == -2 and b"head_dim" in L.qfa_last_error()
+    assert fwd(io=0) == -1 and b"io_dtype" in L.qfa_last_error()
+    rc = L.qfa_bwd_delta(None, ok_ptr, ok_ptr, 2, 1, 1, 8, 64, 512, 512, 64, 512, 512, 64, None)
+    assert rc == -1
+
+
+def test_cpu_tensors_are_refused_not_emulated(qfa):
+    x = torch.randn(1, 2, 16, 64)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        qfa.asymmetric_quant_per_token(x)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        qfa.quant_flash_attn_qkv(x, x, x, False, 0.125)
+    with pytest.raises(ValueError):
+        qfa.asymmetric_quant_per_token(torch.randn(16, 64))
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from quant_flash_attn_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setenv("QFA_LIB", "/nonexistent/libqfa.so")
+    with pytest.raises(RuntimeError, match="not found"):
+        _lib.lib()
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "quant_flash_attn_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".cpp", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), f
+                assert "libqfa_oracle" not in text, f
