@@ -1,0 +1,226 @@
+#!/usr/bin/env python3
+"""Benchmark of the INT8 quantized flash-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all-configs] [--sdpa]
+
+Workload (the configuration the headline metric is quoted on): B=4, H=32, N=4096, D=128, causal,
+bf16 q/k/v drawn N(0,1) plus a per-token mean offset N(0, 0.5), already resident in HBM.
+One step = per-token INT8 quantization of Q and of K (codes, scale, zero point, row sum) followed
+by the attention forward: the whole forward hot path from bf16 q, k, v to bf16 O.
+
+FLOPs follow the reference's convention (compute_flops.py:103-104: forward = 4*B*H*Nq*Nk*D,
+backward = 2.5x forward) with the causal half removed; the un-halved figure is printed too.
+
+The single JSON line printed last carries
+  value        forward TFLOP/s of the whole step (quantize Q, quantize K, attention forward)
+  roofline     the attention forward kernel alone: algorithmic FLOPs per launch / mean launch
+               duration from HIP events recorded around every launch of the timed region
+  cpu_baseline the reference's CPU-runnable path (torch eager quantize + dequantized SDPA,
+               oracle.reference_cpu_path) timed on this machine's host cores on a bounded sample
+plus fwd+bwd, quantizer and kernel-only figures under "extra".
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published dense peaks
+PEAK_INT8_TOPS = 5000.0
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_HBM_GBS = 8000.0
+# HBM bytes per forward launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
+# profiles/); None until measured for the current kernel
+FWD_TRAFFIC_BYTES = None
+
+
+def flops_fwd(B, H, Nq, Nk, D, causal):
+    f = 4.0 * B * H * Nq * Nk * D           # compute_flops.py:103
+    return f * 0.5 if causal else f
+
+
+def time_events(fn, steps, warmup):
+    """Mean milliseconds per call from HIP events on torch's current stream (where fn launches)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(steps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / steps
+
+
+def cpu_baseline(cfg, budget_s=12.0):
+    """Reference CPU path on head-chunks of the same workload until ~budget_s of CPU time."""
+    from oracle import oracle
+    B, H, N, D, causal = cfg["B"], cfg["H"], cfg["N"], cfg["D"], cfg["causal"]
+    sm = 1.0 / math.sqrt(D)
+    threads = torch.get_num_threads()
+    chunk = 4
+    q, k, v, _ = oracle.make_inputs(cfg["dist"], 1, chunk, N, D, seed=1)
+    q, k, v = q.float(), k.float(), v.float()
+    with torch.no_grad():
+        oracle.reference_cpu_path(q[:, :1], k[:, :1], v[:, :1], causal, sm)      # warm-up
+        done, t0 = 0, time.perf_counter()
+        while True:
+            oracle.reference_cpu_path(q, k, v, causal, sm)
+            done += chunk
+            el = time.perf_counter() - t0
+            if el >= budget_s or done >= B * H:
+                break
+    fl = flops_fwd(1, done, N, N, D, causal)
+    return {"value": round(fl / el / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"{done} of {B * H} (batch,head) slices of the same workload, N={N} D={D} "
+                      f"causal={causal}, fp32 torch eager quantize+dequantize+SDPA forward, {el:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--all-configs", action="store_true", help="also time the long-context and D=64 configurations")
+    ap.add_argument("--sdpa", action="store_true", help="also time torch SDPA bf16 on the GPU (stand-in bar)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build is single-GPU by design (every (batch, head) is independent; "
+              "nothing here uses a second GPU). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: needs a GPU", file=sys.stderr)
+        sys.exit(1)
+
+    import quant_flash_attn_amd as qfa
+    from oracle import oracle   # only for synthetic inputs and the CPU-baseline leg
+
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    cfg = {"B": 4, "H": 32, "N": 4096, "D": 128, "causal": True, "dist": "offset"}
+    B, H, N, D, causal = cfg["B"], cfg["H"], cfg["N"], cfg["D"], cfg["causal"]
+    sm = 1.0 / math.sqrt(D)
+    q, k, v, do = (t.to(dev) for t in oracle.make_inputs(cfg["dist"], B, H, N, D, seed=0))
+    F_fwd = flops_fwd(B, H, N, N, D, causal)
+    F_bwd = 2.5 * F_fwd                       # compute_flops.py:104
+
+    # ---- the timed region: K steps of (quantize Q, quantize K, forward), wall clock, with HIP
+    # events around every attention launch for the kernel's own duration
+    def step(evs=None):
+        qq = qfa.quantize_for_attention(q)
+        kq = qfa.quantize_for_attention(k)
+        if evs is not None:
+            evs[0].record()
+        o, lse = qfa.attn_fwd_quantized(qq, kq, v, causal, sm)
+        if evs is not None:
+            evs[1].record()
+        return qq, kq, o, lse
+
+    for _ in range(args.warmup):
+        step()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        qq, kq, o, lse = step(events[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_step = (t1 - t0) * 1e3 / args.steps
+    ms_fwd_kernel = sum(a.elapsed_time(b) for a, b in events) / args.steps
+    value = F_fwd / (ms_step * 1e-3) / 1e12
+
+    # ---- extras (outside the timed region)
+    extra = {}
+    ms_quant = time_events(lambda: qfa.quantize_for_attention(q), 50, 10)
+    tok = B * H * N
+    quant_bytes = tok * (D * 2 + D + 4 + 1 + 4)          # bf16 in; codes, fp32 scale, zp, rowsum out
+    extra["quant_ms_per_tensor"] = round(ms_quant, 4)
+    extra["quant_GBps"] = round(quant_bytes / (ms_quant * 1e-3) / 1e9, 1)
+    extra["quant_frac_hbm_peak"] = round(quant_bytes / (ms_quant * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)
+    ms_fwd_only = time_events(lambda: qfa.attn_fwd_quantized(qq, kq, v, causal, sm), args.steps, 5)
+    extra["fwd_kernel_ms"] = round(ms_fwd_only, 4)
+    extra["fwd_kernel_tflops"] = round(F_fwd / (ms_fwd_only * 1e-3) / 1e12, 2)
+    extra["fwd_kernel_tflops_unhalved_formula"] = round(2 * F_fwd / (ms_fwd_only * 1e-3) / 1e12, 2)
+    ms_bwd = time_events(lambda: qfa.attn_bwd_quantized(qq, kq, v, o, do, lse, causal, sm), max(5, args.steps // 2), 3)
+    extra["bwd_ms"] = round(ms_bwd, 4)
+    extra["bwd_tflops"] = round(F_bwd / (ms_bwd * 1e-3) / 1e12, 2)
+    extra["fwd_bwd_ms_incl_quant"] = round(ms_step + ms_bwd, 4)
+    extra["fwd_bwd_tflops_incl_quant"] = round((F_fwd + F_bwd) / ((ms_step + ms_bwd) * 1e-3) / 1e12, 2)
+    extra["fwd_bwd_tflops_kernels_only"] = round((F_fwd + F_bwd) / ((ms_fwd_only + ms_bwd) * 1e-3) / 1e12, 2)
+    # the QK^T product is half of the forward FLOPs and runs on INT8 MFMA
+    extra["qk_int8_tops_over_whole_fwd_kernel"] = round(0.5 * F_fwd / (ms_fwd_only * 1e-3) / 1e12, 2)
+    extra["qk_frac_int8_peak_over_whole_fwd_kernel"] = round(0.5 * F_fwd / (ms_fwd_only * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)
+
+    if args.sdpa:
+        import torch.nn.functional as Fn
+        qs, ks, vs = (t.clone().requires_grad_(True) for t in (q, k, v))
+        ms_s = time_events(lambda: Fn.scaled_dot_product_attention(qs.detach(), ks.detach(), vs.detach(), is_causal=causal, scale=sm), 20, 5)
+        extra["torch_sdpa_bf16_fwd_ms"] = round(ms_s, 4)
+        extra["torch_sdpa_bf16_fwd_tflops"] = round(F_fwd / (ms_s * 1e-3) / 1e12, 2)
+
+        def fb():
+            out = Fn.scaled_dot_product_attention(qs, ks, vs, is_causal=causal, scale=sm)
+            out.backward(do)
+            qs.grad = ks.grad = vs.grad = None
+        ms_sb = time_events(fb, 10, 3)
+        extra["torch_sdpa_bf16_fwd_bwd_ms"] = round(ms_sb, 4)
+        extra["torch_sdpa_bf16_fwd_bwd_tflops"] = round((F_fwd + F_bwd) / (ms_sb * 1e-3) / 1e12, 2)
+
+    if args.all_configs:
+        others = {"long_context_B1_H16_N16384_D128_noncausal": (1, 16, 16384, 128, False, "outlier"),
+                  "small_head_B16_H16_N2048_D64_causal": (16, 16, 2048, 64, True, "uniform")}
+        del q, k, v, do, qq, kq, o, lse
+        for name, (b2, h2, n2, d2, c2, dist) in others.items():
+            q2, k2, v2, do2 = (t.to(dev) for t in oracle.make_inputs(dist, b2, h2, n2, d2, seed=0))
+            sm2 = 1.0 / math.sqrt(d2)
+            f2 = flops_fwd(b2, h2, n2, n2, d2, c2)
+            qq2, kq2 = qfa.quantize_for_attention(q2), qfa.quantize_for_attention(k2)
+            o2, lse2 = qfa.attn_fwd_quantized(qq2, kq2, v2, c2, sm2)
+            mq = time_events(lambda: qfa.quantize_for_attention(q2), 30, 5)
+            mf = time_events(lambda: qfa.attn_fwd_quantized(qq2, kq2, v2, c2, sm2), 20, 3)
+            mb = time_events(lambda: qfa.attn_bwd_quantized(qq2, kq2, v2, o2, do2, lse2, c2, sm2), 10, 2)
+            qb = b2 * h2 * n2 * (d2 * 2 + d2 + 9)
+            extra[name] = {"fwd_ms": round(mf, 4), "fwd_tflops": round(f2 / mf / 1e9, 2), "bwd_ms": round(mb, 4),
+                           "bwd_tflops": round(2.5 * f2 / mb / 1e9, 2),
+                           "fwd_bwd_tflops": round(3.5 * f2 / (mf + mb) / 1e9, 2),
+                           "quant_ms_per_tensor": round(mq, 4), "quant_GBps": round(qb / mq / 1e6, 1)}
+            del q2, k2, v2, do2, qq2, kq2, o2, lse2
+
+    # ---- roofline of the dominant kernel (attention forward): half its FLOPs are INT8 (QK^T), half
+    # bf16 (P.V), so the MFMA time floor is F/2/P_int8 + F/2/P_bf16 and the peak it is priced
+    # against is the harmonic blend of the two published peaks
+    peak_blend = 2.0 / (1.0 / PEAK_INT8_TOPS + 1.0 / PEAK_BF16_TFLOPS)
+    achieved = F_fwd / (ms_fwd_kernel * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": "fwd_kernel<bf16,128,causal>", "achieved": round(achieved, 2),
+                "peak": round(peak_blend, 1), "unit": "TFLOP/s", "frac": round(achieved / peak_blend, 4),
+                "traffic": FWD_TRAFFIC_BYTES, "algorithmic_flops_per_launch": F_fwd,
+                "mean_launch_ms": round(ms_fwd_kernel, 4),
+                "frac_of_bf16_peak": round(achieved / PEAK_BF16_TFLOPS, 4),
+                "peak_note": "harmonic blend of published dense INT8 (5.0 POP/s, QK^T half) and bf16 (2.5 PFLOP/s, PV half)"}
+
+    result = {
+        "metric": "attn TFLOPS fwd & fwd+bwd @B4 H32 N4096 D128 causal; % of INT8 MFMA peak",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 (QK^T, int32 accumulate) + bf16 (P.V) + fp32 softmax", "data": "synthetic",
+        "config": {"workload": "forward causal B=4 H=32 N=4096 D=128 bf16: quantize Q, quantize K, attention forward",
+                   "flops_convention": "4*B*H*N*N*D/2 (compute_flops.py:103, causal-halved)"},
+        "roofline": roofline,
+        "cpu_baseline": None if args.no_cpu else cpu_baseline(cfg),
+        "extra": extra,
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

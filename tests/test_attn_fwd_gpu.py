@@ -114,7 +114,7 @@ def test_key_permutation_invariance(qfa):
     _, _, o, lse = _run(qfa, q, k, v, False, sm)
     perm = torch.randperm(512, generator=torch.Generator().manual_seed(1))
     _, _, o_p, lse_p = _run(qfa, q, k[:, :, perm], v[:, :, perm], False, sm)
-    assert max_abs(o, o_p) < 8e-3 and max_abs(lse, lse_p) < 1e-4
+    assert max_abs(o, o_p) <= 2e-2 and max_abs(lse, lse_p) < 1e-4   # O within two bf16 ulps of |O| <= 4
 
 
 def test_output_fully_written_and_deterministic(qfa):
