@@ -93,6 +93,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--all-configs", action="store_true", help="also time the long-context and D=64 configurations")
     ap.add_argument("--sdpa", action="store_true", help="also time torch SDPA bf16 on the GPU (stand-in bar)")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run a plain 256 MiB device-to-device copy (calibrates rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build is single-GPU by design (every (batch, head) is independent; "
@@ -141,6 +143,13 @@ def main():
 
     # ---- extras (outside the timed region)
     extra = {}
+    if args.calib_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     ms_quant = time_events(lambda: qfa.quantize_for_attention(q), 50, 10)
     tok = B * H * N
     quant_bytes = tok * (D * 2 + D + 4 + 1 + 4)          # bf16 in; codes, fp32 scale, zp, rowsum out
