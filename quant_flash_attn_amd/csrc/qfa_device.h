@@ -52,6 +52,17 @@ template <typename T> __device__ __forceinline__ float hi_to_f32(unsigned w) {
   return (float)q[1];
 }
 
+// c + lo(w) + hi(w) for a packed pair of 16-bit floats (v_dot2 with a pair of ones), fp32 accumulate
+template <typename T> __device__ __forceinline__ float dot2_ones(unsigned w, float c);
+template <> __device__ __forceinline__ float dot2_ones<__bf16>(unsigned w, float c) {
+  const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), ones, c, false);
+}
+template <> __device__ __forceinline__ float dot2_ones<_Float16>(unsigned w, float c) {
+  const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), ones, c, false);
+}
+
 // ---- MFMA wrappers (A and B: 16 bytes per lane; C/D: 16 dwords per lane) ------------------------
 // 32x32x32 int8:  A lane l = row l%32, 16 consecutive k at k-group l/32;  B lane l = column l%32,
 // same k slots;  D lane l = column l%32, register v = row 8*(v/4) + 4*(l/32) + v%4.

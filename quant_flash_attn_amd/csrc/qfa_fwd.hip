@@ -2,8 +2,8 @@
 // INT8 codes (scale, zero point, row sum per token).  gfx950, wave64.
 //
 // Work split.  One workgroup = 4 waves = 128 query rows of one (batch, head); each wave owns
-// 32 queries.  K/V stream through LDS in tiles of 64 keys, double buffered (global -> registers
-// while the previous tile is being consumed, registers -> LDS afterwards, one barrier per tile).
+// 32 queries.  K (3 buffers) and V (2 buffers) stream through LDS in tiles of 64 keys: K and the
+// per-key constants are resident one tile ahead of V because the score product runs ahead.
 //
 // Score tile.  Each wave computes S^T = Kc . Qc^T with v_mfma_i32_32x32x32_i8: the K rows come
 // from LDS (A operand), the wave's 32 queries stay in registers for the whole kernel (B operand).
@@ -13,13 +13,28 @@
 // O^T = V^T . P^T (v_mfma_f32_32x32x16_bf16/f16) without leaving registers.
 //
 // Zero points.  With integer codes,  sum_d (qc-zq)(kc-zk) = A - zq*rk - zk*(rq - D*zq), A the int32
-// MFMA result and rq, rk the code row sums.  The two corrections are applied as exact fp32 FMAs on
-// the converted accumulator (every intermediate is an integer below 2^24), then one multiply by
-// the key scale; the query scale, sm_scale and log2(e) are folded into the exp2 argument.
+// MFMA result and rq, rk the code row sums.  The correction is a rank-4 update with integer
+// entries below 2^8 (rk and rq - D*zq split into base-128 digits), so it runs as ONE extra 16-bit
+// MFMA on the converted accumulator instead of per-score VALU work; every product and partial sum
+// is an integer below 2^24, hence exact in fp32.  Then one multiply by the key scale; the query
+// scale, sm_scale and log2(e) are folded into the exp2 argument.
+//
+// The kernel is bound by softmax VALU work, not by MFMA, so the design goal is to keep the vector
+// pipe busy and hide the matrix pipe under it:
+//  * the running maximum is only moved (and O rescaled) when some row of the wave exceeds it by
+//    more than 2^8 (any reference maximum gives the same O after the final division), so the
+//    rescale is a rare branch instead of 64 multiplies per tile;
+//  * row sums are taken over packed pairs with v_dot2;
+//  * tiles without any masked score run a software-pipelined loop whose body is one straight
+//    basic block per 32-key block: exp2/pack of block b, the P.V MFMAs of block b, the INT8 MFMAs
+//    of block b+2 and the convert/correct/scale/max of block b+1 are independent of each other,
+//    so MFMA and VALU instructions interleave; diagonal and ragged tiles run a simple masked loop.
 //
 // V is transposed on its way into LDS (Vt[d][key]) so a lane reads its 8 keys of one d as one
 // 16-byte LDS load; keys are stored in the permuted order in which the S^T accumulator layout
 // hands out P, so no shuffle is needed between the two products.
+#include <type_traits>
+
 #include "qfa_device.h"
 #include "qfa_host.h"
 
@@ -40,15 +55,25 @@ struct FwdArgs {
 
 constexpr int FWD_BM = 128;
 constexpr int FWD_BN = 64;
+constexpr float FWD_RESCALE_THRESHOLD = 8.0f;   // log2 units the running max may lag behind
 
 template <int D> struct FwdSmem {
   static constexpr int KSTR = D + 16;            // bytes per K row (+16: conflict-free 16-byte reads)
   static constexpr int VSTR = (FWD_BN + 8) * 2;  // bytes per Vt row
   static constexpr int K_BYTES = FWD_BN * KSTR;
   static constexpr int V_BYTES = D * VSTR;
-  static constexpr int C_BYTES = 3 * FWD_BN * 4;  // sk, float(rk), float(zk)
-  static constexpr int BUF_BYTES = K_BYTES + V_BYTES + C_BYTES;
+  static constexpr int C_BYTES = FWD_BN * 4 + FWD_BN * 8;  // key scale; correction digits (2 dwords/key)
+  static constexpr int OFF_K = 0;                     // 3 buffers
+  static constexpr int OFF_V = 3 * K_BYTES;           // 2 buffers
+  static constexpr int OFF_C = OFF_V + 2 * V_BYTES;   // 3 buffers
+  static constexpr int TOTAL = OFF_C + 3 * C_BYTES;
 };
+
+// integer n in [-32768, 32767] -> (128*floor(n/128), n mod 128) as a packed pair of 16-bit floats
+template <typename T> __device__ __forceinline__ unsigned base128_pair(int n) {
+  const int hi = n >> 7, lo = n & 127;
+  return pack2<T>((float)(hi * 128), (float)lo);
+}
 
 template <typename T, int D, bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
@@ -56,7 +81,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
   constexpr int KS = D / 32;   // int8 k-steps of 32
   constexpr int DB = D / 32;   // 32-row blocks of O^T
   constexpr int KCH = (FWD_BN * D / 16) / 256;   // 16-byte K chunks per thread (2 for D=128, 1 for D=64)
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * SM::BUF_BYTES];
+  __shared__ __attribute__((aligned(16))) unsigned char smem[SM::TOTAL];
 
   // ---- block -> (batch*head, query block); consecutive ids of one XCD share a head's K/V in its L2
   const int L = blockIdx.x;
@@ -88,10 +113,16 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
     qf[ks] = *reinterpret_cast<const i32x4 *>(qc_bh + (int64_t)qi_c * a.sqn + ks * 32 + g * 16);
-  const float zqf = (float)a.zq[tq0 + qi_c];
+  const int zq_i = (int)a.zq[tq0 + qi_c];
   const float a_i = a.sq[tq0 + qi_c] * a.sm_scale_log2;        // > 0
-  const float nzq = -zqf;
-  const float nc = -((float)a.rq[tq0 + qi_c] - (float)D * zqf);  // exact: |.| < 2^16
+  // query side of the rank-4 correction: k-group 0 multiplies the two digits of rk by -zq,
+  // k-group 1 multiplies zk (stored twice) by minus the two digits of c = rq - D*zq
+  u32x4 corr_q = {0u, 0u, 0u, 0u};
+  {
+    const int c = a.rq[tq0 + qi_c] - D * zq_i;     // |c| <= 32640
+    const int hi = c >> 7, lo = c & 127;
+    corr_q[0] = g == 0 ? pack2<T>((float)(-zq_i), (float)(-zq_i)) : pack2<T>((float)(-128 * hi), (float)(-lo));
+  }
   const int q_first = m0 + wave * 32, q_last = q_first + 31;
 
   // ---- tile range
@@ -107,9 +138,10 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
 
   u32x4 kreg[KCH];
   u32x4 vreg[4];
-  float creg[3];
+  float c_sk;
+  int c_rk, c_zk;
 
-  auto load_tile = [&](int t) {
+  auto load_k = [&](int t) {
     const int j0 = t * FWD_BN;
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
@@ -118,6 +150,32 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
       const int j = min(j0 + row, a.Nk - 1);
       kreg[i] = *reinterpret_cast<const u32x4 *>(kc_bh + (int64_t)j * a.skn + col * 16);
     }
+    if (tid < FWD_BN) {
+      const int j = min(j0 + tid, a.Nk - 1);
+      c_sk = a.sk[tk0 + j];
+      c_rk = a.rk[tk0 + j];
+      c_zk = (int)a.zk[tk0 + j];
+    }
+  };
+  auto store_k = [&](int buf) {
+    unsigned char *base = smem + SM::OFF_K + buf * SM::K_BYTES;
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c / (D / 16), col = c % (D / 16);
+      *reinterpret_cast<u32x4 *>(base + row * SM::KSTR + col * 16) = kreg[i];
+    }
+    if (tid < FWD_BN) {
+      unsigned char *cb = smem + SM::OFF_C + buf * SM::C_BYTES;
+      reinterpret_cast<float *>(cb)[tid] = c_sk;
+      u32x2 dg;
+      dg[0] = base128_pair<T>(c_rk);                      // k-group 0: digits of rk
+      dg[1] = pack2<T>((float)c_zk, (float)c_zk);         // k-group 1: zk, zk
+      reinterpret_cast<u32x2 *>(cb + FWD_BN * 4)[tid] = dg;
+    }
+  };
+  auto load_v = [&](int t) {
+    const int j0 = t * FWD_BN;
     if (v_active) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -125,23 +183,10 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
         vreg[r] = *reinterpret_cast<const u32x4 *>(v_bh + (int64_t)j * a.svn + v_dc * 8);
       }
     }
-    if (tid < FWD_BN) {
-      const int j = min(j0 + tid, a.Nk - 1);
-      creg[0] = a.sk[tk0 + j];
-      creg[1] = (float)a.rk[tk0 + j];
-      creg[2] = (float)a.zk[tk0 + j];
-    }
   };
-  auto store_tile = [&](int buf) {
-    unsigned char *base = smem + buf * SM::BUF_BYTES;
-#pragma unroll
-    for (int i = 0; i < KCH; ++i) {
-      const int c = tid + 256 * i;
-      const int row = c / (D / 16), col = c % (D / 16);
-      *reinterpret_cast<u32x4 *>(base + row * SM::KSTR + col * 16) = kreg[i];
-    }
+  auto store_v = [&](int buf) {
     if (v_active) {
-      unsigned char *vt = base + SM::K_BYTES;
+      unsigned char *vt = smem + SM::OFF_V + buf * SM::V_BYTES;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {   // d = 8*v_dc + e: gather the 4 keys of that d
         const int w = e / 2;
@@ -156,11 +201,16 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
         *reinterpret_cast<u32x2 *>(vt + (v_dc * 8 + e) * SM::VSTR + v_pos * 2) = o;
       }
     }
-    if (tid < FWD_BN) {
-      float *cs = reinterpret_cast<float *>(base + SM::K_BYTES + SM::V_BYTES);
-      cs[tid] = creg[0];
-      cs[FWD_BN + tid] = creg[1];
-      cs[2 * FWD_BN + tid] = creg[2];
+  };
+  // S^T block nb (32 keys) of the tile held in K buffer `buf`, for this wave's 32 queries
+  auto qk_block = [&](int buf, int nb, i32x16 &s) {
+    const unsigned char *ks_ = smem + SM::OFF_K + buf * SM::K_BYTES;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const i32x4 kf = *reinterpret_cast<const i32x4 *>(ks_ + (32 * nb + lr) * SM::KSTR + ks * 32 + g * 16);
+      s = mfma_i8(kf, qf[ks], s);
     }
   };
 
@@ -169,98 +219,141 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int v = 0; v < 16; ++v) oacc[db][v] = 0.f;
-  float m_run = -INFINITY;   // running max of u = score / a_i
+  float m_ref = -INFINITY;   // reference maximum of u = score / a_i used in the exponent
+  float nm = INFINITY;       // -a_i * m_ref
   float l_run = 0.f;         // this lane's share of the row sum
 
-  load_tile(0);
-  store_tile(0);
+  // raw int32 block -> u = sk * (S + zero-point correction); returns the block maximum of the row
+  auto prep = [&](int cbuf, int nb, const i32x16 &s, float (&u)[16], int j0, auto masked_tag) -> float {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    const unsigned char *cb = smem + SM::OFF_C + cbuf * SM::C_BYTES;
+    const float *skp = reinterpret_cast<const float *>(cb);
+    const unsigned *dgp = reinterpret_cast<const unsigned *>(cb + FWD_BN * 4);
+    f32x16 f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
+    u32x4 corr_k = {dgp[2 * (32 * nb + lr) + g], 0u, 0u, 0u};
+    f = mfma_16b<T>(corr_k, corr_q, f);
+    float mt = -INFINITY;
+#pragma unroll
+    for (int aa = 0; aa < 4; ++aa) {
+      const int jl = 32 * nb + 8 * aa + 4 * g;
+      const f32x4 sk4 = *reinterpret_cast<const f32x4 *>(skp + jl);
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) {
+        float uu = f[4 * aa + bb] * sk4[bb];
+        if (MASKED) {
+          const int j = j0 + jl + bb;
+          if ((CAUSAL && j > qi) || j >= a.Nk) uu = -INFINITY;
+        }
+        u[4 * aa + bb] = uu;
+        mt = fmaxf(mt, uu);
+      }
+    }
+    return fmaxf(mt, swap32_f(mt));
+  };
+  // move the reference maximum only when some row of the wave outgrew it by > 2^threshold
+  auto rescale_if_needed = [&](float mt) {
+    if (__builtin_amdgcn_ballot_w64(a_i * (mt - m_ref) > FWD_RESCALE_THRESHOLD) != 0) {
+      const float m_new = fmaxf(m_ref, mt);
+      const float alpha = __builtin_amdgcn_exp2f(a_i * (m_ref - m_new));
+      m_ref = m_new;
+      nm = -a_i * m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) oacc[db][v] *= alpha;
+    }
+  };
+  // p = exp2(a_i*u - a_i*m_ref), packed; row sum; O^T += V^T . P^T for the 32 keys of block nb
+  auto exp_pv = [&](int vbuf, int nb, const float (&u)[16]) {
+    const unsigned char *vt_ = smem + SM::OFF_V + vbuf * SM::V_BYTES;
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      u32x4 pf;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, u[8 * hh + 2 * e], nm));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, u[8 * hh + 2 * e + 1], nm));
+        pf[e] = pack2<T>(p0, p1);
+        l_run = dot2_ones<T>(pf[e], l_run);   // sum of the rounded pair, fp32 accumulate
+      }
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const u32x4 vf =
+            *reinterpret_cast<const u32x4 *>(vt_ + (32 * db + lr) * SM::VSTR + (32 * nb + 16 * hh + 8 * g) * 2);
+        oacc[db] = mfma_16b<T>(vf, pf, oacc[db]);
+      }
+    }
+  };
+
+  // ---- prologue: K(0), K(1) (with their constants) and V(0) resident
+  load_k(0);
+  load_v(0);
+  store_k(0);
+  store_v(0);
+  if (ntiles > 1) {
+    load_k(1);
+    store_k(1);
+  }
   __syncthreads();
 
-  for (int t = 0; t < ntiles; ++t) {
-    const int buf = t & 1;
-    if (t + 1 < ntiles) load_tile(t + 1);
+  // tiles [0, t_hot) contain no masked score for this wave (wave-uniform)
+  int t_hot = a.Nk / FWD_BN;
+  if (CAUSAL) t_hot = min(t_hot, (q_first + 1) / FWD_BN);
+  t_hot = min(t_hot, ntiles);
 
-    const unsigned char *base = smem + buf * SM::BUF_BYTES;
-    const unsigned char *ks_ = base;
-    const unsigned char *vt_ = base + SM::K_BYTES;
-    const float *cs = reinterpret_cast<const float *>(base + SM::K_BYTES + SM::V_BYTES);
+  int kb_cur = 0, kb_nxt = 1, kb_free = 2;   // K/constant buffers of tile t, t+1, and the one to refill
+  int t = 0;
+  {
+    // ---- pipelined loop over unmasked tiles.  Entering tile t: u_a = prepared block 2t,
+    // s_y = raw S of block 2t+1; the reference maximum already covers block 2t.
+    float u_a[16], u_b[16];
+    i32x16 s_x, s_y;
+    if (t_hot > 0) {
+      qk_block(0, 0, s_x);
+      qk_block(0, 1, s_y);
+      rescale_if_needed(prep(0, 0, s_x, u_a, 0, std::false_type{}));
+    }
+    for (; t < t_hot; ++t) {
+      if (t + 2 < ntiles) load_k(t + 2);
+      if (t + 1 < ntiles) load_v(t + 1);
+      // block 2t: consume u_a; raw S(2t+2) -> s_x; prepare block 2t+1 from s_y
+      qk_block(kb_nxt, 0, s_x);
+      exp_pv(t & 1, 0, u_a);
+      rescale_if_needed(prep(kb_cur, 1, s_y, u_b, 0, std::false_type{}));
+      // block 2t+1: consume u_b; raw S(2t+3) -> s_y; prepare block 2t+2 from s_x (only a
+      // candidate maximum if that block belongs to the unmasked range)
+      qk_block(kb_nxt, 1, s_y);
+      exp_pv(t & 1, 1, u_b);
+      const float mt = prep(kb_nxt, 0, s_x, u_a, 0, std::false_type{});
+      rescale_if_needed(t + 1 < t_hot ? mt : -INFINITY);
+
+      if (t + 2 < ntiles) store_k(kb_free);
+      if (t + 1 < ntiles) store_v((t + 1) & 1);
+      const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
+      __syncthreads();
+    }
+  }
+  // ---- masked tiles (diagonal, ragged end): one block at a time, nothing carried between blocks
+  for (; t < ntiles; ++t) {
+    if (t + 2 < ntiles) load_k(t + 2);
+    if (t + 1 < ntiles) load_v(t + 1);
     const int j0 = t * FWD_BN;
-
-    bool blk_on[2];
-    float u[2][16];
-    float mt = -INFINITY;
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
       const int jb = j0 + 32 * nb;
-      blk_on[nb] = (jb < a.Nk) && (!CAUSAL || jb <= q_last);   // wave-uniform
-      if (!blk_on[nb]) continue;
-      i32x16 acc;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[v] = 0;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const i32x4 kf = *reinterpret_cast<const i32x4 *>(ks_ + (32 * nb + lr) * SM::KSTR + ks * 32 + g * 16);
-        acc = mfma_i8(kf, qf[ks], acc);
-      }
-      const bool need_mask = (CAUSAL && jb + 31 > q_first) || (jb + 32 > a.Nk);   // wave-uniform
-#pragma unroll
-      for (int aa = 0; aa < 4; ++aa) {
-        const int jl = 32 * nb + 8 * aa + 4 * g;
-        const f32x4 sk4 = *reinterpret_cast<const f32x4 *>(cs + jl);
-        const f32x4 rk4 = *reinterpret_cast<const f32x4 *>(cs + FWD_BN + jl);
-        const f32x4 zk4 = *reinterpret_cast<const f32x4 *>(cs + 2 * FWD_BN + jl);
-#pragma unroll
-        for (int bb = 0; bb < 4; ++bb) {
-          float f = (float)acc[4 * aa + bb];
-          f = __builtin_fmaf(nzq, rk4[bb], f);
-          f = __builtin_fmaf(nc, zk4[bb], f);
-          float uu = f * sk4[bb];
-          if (need_mask) {
-            const int j = j0 + jl + bb;
-            if ((CAUSAL && j > qi) || j >= a.Nk) uu = -INFINITY;
-          }
-          u[nb][4 * aa + bb] = uu;
-          mt = fmaxf(mt, uu);
-        }
-      }
+      if ((CAUSAL && jb > q_last) || jb >= a.Nk) continue;   // wave-uniform: nothing to keep
+      i32x16 s;
+      float u[16];
+      qk_block(kb_cur, nb, s);
+      rescale_if_needed(prep(kb_cur, nb, s, u, j0, std::true_type{}));
+      exp_pv(t & 1, nb, u);
     }
-    mt = fmaxf(mt, swap32_f(mt));
-    const float m_new = fmaxf(m_run, mt);
-    const float alpha = __builtin_amdgcn_exp2f(a_i * (m_run - m_new));
-    const float nm = -a_i * m_new;
-    m_run = m_new;
-    l_run *= alpha;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) oacc[db][v] *= alpha;
-
-#pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
-      if (!blk_on[nb]) continue;
-      float psum = 0.f;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, u[nb][v], nm));
-        u[nb][v] = p;
-        psum += p;
-      }
-      l_run += psum;
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
-        u32x4 pf;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) pf[e] = pack2<T>(u[nb][8 * hh + 2 * e], u[nb][8 * hh + 2 * e + 1]);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const u32x4 vf =
-              *reinterpret_cast<const u32x4 *>(vt_ + (32 * db + lr) * SM::VSTR + (32 * nb + 16 * hh + 8 * g) * 2);
-          oacc[db] = mfma_16b<T>(vf, pf, oacc[db]);
-        }
-      }
-    }
-
-    if (t + 1 < ntiles) store_tile(buf ^ 1);
+    if (t + 2 < ntiles) store_k(kb_free);
+    if (t + 1 < ntiles) store_v((t + 1) & 1);
+    const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
     __syncthreads();
   }
 
@@ -278,7 +371,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
         w[1] = pack2<T>(oacc[db][4 * aa + 2] * inv, oacc[db][4 * aa + 3] * inv);
         *reinterpret_cast<u32x2 *>(orow + 32 * db + 8 * aa + 4 * g) = w;
       }
-    if (g == 0) a.lse[tq0 + qi] = (a_i * m_run + __log2f(l_tot)) * kLn2;
+    if (g == 0) a.lse[tq0 + qi] = (a_i * m_ref + __log2f(l_tot)) * kLn2;
   }
 }
 

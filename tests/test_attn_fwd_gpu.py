@@ -12,6 +12,7 @@ from oracle import oracle
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
+LSE_TOL = 2.0 ** -8   # row sums are taken over the 16-bit-rounded probabilities (2^-9 relative each)
 
 
 def _run(qfa, q, k, v, causal, sm):
@@ -55,7 +56,7 @@ def test_forward_vs_oracle(qfa, B, H, Nq, Nk, D, causal, config, dtype):
     o_ref, lse_ref = _oracle_fwd(qq, kq, v, causal, sm)
     assert o.dtype == dtype and o.shape == (B, H, Nq, D) and lse.shape == (B, H, Nq)
     assert_close("O", o.cpu(), o_ref)
-    assert max_abs(lse.cpu(), lse_ref) < 1e-3
+    assert max_abs(lse.cpu(), lse_ref) < LSE_TOL
     # the quantized inputs the kernel consumed are the oracle's
     assert torch.equal(qq.codes.cpu(), oracle.quantize_per_token_c(q)[0])
 
@@ -94,7 +95,7 @@ def test_full_size_sampled_heads_and_properties(qfa, config, B, H, N, D, causal)
             s = s.masked_fill(torch.arange(N)[None, :] > i, float("-inf"))
         o_ref = torch.softmax(s, -1) @ sel(v).double()
         assert_close(f"O[{b},{h}]", o.cpu()[b:b + 1, h:h + 1, rows], o_ref)
-        assert max_abs(lse.cpu()[b:b + 1, h:h + 1, rows], torch.logsumexp(s, -1)) < 1e-3
+        assert max_abs(lse.cpu()[b:b + 1, h:h + 1, rows], torch.logsumexp(s, -1)) < LSE_TOL
     if causal:   # row 0 only sees key 0
         assert torch.equal(o[:, :, 0], v.to(DEV)[:, :, 0])
     # rows of P sum to one: with V = 1 the output is 1 (up to the 16-bit rounding of P)
@@ -114,7 +115,7 @@ def test_key_permutation_invariance(qfa):
     _, _, o, lse = _run(qfa, q, k, v, False, sm)
     perm = torch.randperm(512, generator=torch.Generator().manual_seed(1))
     _, _, o_p, lse_p = _run(qfa, q, k[:, :, perm], v[:, :, perm], False, sm)
-    assert max_abs(o, o_p) <= 2e-2 and max_abs(lse, lse_p) < 1e-4   # O within two bf16 ulps of |O| <= 4
+    assert max_abs(o, o_p) <= 2e-2 and max_abs(lse, lse_p) < 2 * LSE_TOL   # O within two bf16 ulps of |O| <= 4
 
 
 def test_output_fully_written_and_deterministic(qfa):
