@@ -94,7 +94,8 @@ int qfa_attn_fwd(const int8_t *qc, const float *sq, const int8_t *zq, const int3
 /*
  * delta[b,h,n] = sum_d O[b,h,n,d] * dO[b,h,n,d], accumulated in fp32.
  * Replaces the launch of _bwd_preprocess_kernel (quant_flash_attn.py:87-101, :217-223).
- * qfa_attn_bwd calls this itself; it is exported for callers that split the backward.
+ * qfa_attn_bwd computes delta inside its own staging pass; this entry point is for callers that
+ * only need the preprocess step.
  */
 int qfa_bwd_delta(const void *o, const void *dout, float *delta, int io_dtype, int64_t B, int64_t H, int64_t N,
                   int D, int64_t sob, int64_t soh, int64_t son, int64_t sdb, int64_t sdh, int64_t sdn,
@@ -106,12 +107,18 @@ int qfa_bwd_delta(const void *o, const void *dout, float *delta, int io_dtype, i
  *                 dQ = sm_scale dS K^,  dK = sm_scale dS^T Q^      (gradients w.r.t. Q^, K^).
  * Replaces the launches made by QuantFlashAttention.backward (quant_flash_attn.py:104-166
  * kernel, :207-237 wrapper); the reference's single dKV tensor is dK + dV (:161).
- *   delta  float [B*H*Nq] workspace, overwritten.
+ *   workspace  caller-owned scratch of at least qfa_attn_bwd_workspace_bytes(B,H,Nq,Nk,D) bytes,
+ *              16-byte aligned, overwritten: two staging passes fill it with delta = rowsum(O o dO),
+ *              the transposed 16-bit tiles dO^T, (Qc-zq)^T, (Kc-zk)^T and per-token constants, once
+ *              per call, so that the two MFMA kernels stream ready-made tiles.
  *   dq [B,H,Nq,D], dk, dv [B,H,Nk,D] of io_dtype, strides as given.
  */
+int64_t qfa_attn_bwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D);
+
 int qfa_attn_bwd(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,
                  const float *sk, const int8_t *zk, const int32_t *rk, const void *v, const void *o,
-                 const void *dout, const float *lse, float *delta, void *dq, void *dk, void *dv, int io_dtype,
+                 const void *dout, const float *lse, void *workspace, int64_t workspace_bytes, void *dq, void *dk,
+                 void *dv, int io_dtype,
                  int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D, int64_t sqb, int64_t sqh, int64_t sqn,
                  int64_t skb, int64_t skh, int64_t skn, int64_t svb, int64_t svh, int64_t svn, int64_t sob,
                  int64_t soh, int64_t son, int64_t sdob, int64_t sdoh, int64_t sdon, int64_t sdqb, int64_t sdqh,

@@ -130,9 +130,15 @@ int qfa_bwd_delta(const void *o, const void *dout, float *delta, int io_dtype, i
   return launch_delta(o, dout, delta, io_dtype, B, H, N, D, sob, soh, son, sdb, sdh, sdn, (hipStream_t)stream);
 }
 
+int64_t qfa_attn_bwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D) {
+  if (B <= 0 || H <= 0 || Nq <= 0 || Nk <= 0 || (D != 64 && D != 128)) return 0;
+  return bwd_workspace_bytes(B, H, Nq, Nk, D);
+}
+
 int qfa_attn_bwd(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,
                  const float *sk, const int8_t *zk, const int32_t *rk, const void *v, const void *o,
-                 const void *dout, const float *lse, float *delta, void *dq, void *dk, void *dv, int io_dtype,
+                 const void *dout, const float *lse, void *workspace, int64_t workspace_bytes, void *dq, void *dk,
+                 void *dv, int io_dtype,
                  int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D, int64_t sqb, int64_t sqh, int64_t sqn,
                  int64_t skb, int64_t skh, int64_t skn, int64_t svb, int64_t svh, int64_t svn, int64_t sob,
                  int64_t soh, int64_t son, int64_t sdob, int64_t sdoh, int64_t sdon, int64_t sdqb, int64_t sdqh,
@@ -142,7 +148,7 @@ int qfa_attn_bwd(const int8_t *qc, const float *sq, const int8_t *zq, const int3
   memset(&a, 0, sizeof(a));
   a.qc = qc; a.sq = sq; a.zq = zq; a.rq = rq; a.kc = kc; a.sk = sk; a.zk = zk; a.rk = rk;
   a.v = v; a.o = const_cast<void *>(o); a.lse = const_cast<float *>(lse); a.io_dtype = io_dtype;
-  a.dout = dout; a.delta = delta; a.dq = dq; a.dk = dk; a.dv = dv;
+  a.dout = dout; a.workspace = workspace; a.dq = dq; a.dk = dk; a.dv = dv;
   a.B = B; a.H = H; a.Nq = Nq; a.Nk = Nk; a.D = D;
   a.sqb = sqb; a.sqh = sqh; a.sqn = sqn; a.skb = skb; a.skh = skh; a.skn = skn;
   a.svb = svb; a.svh = svh; a.svn = svn; a.sob = sob; a.soh = soh; a.son = son;
@@ -150,14 +156,16 @@ int qfa_attn_bwd(const int8_t *qc, const float *sq, const int8_t *zq, const int3
   a.sdkb = sdkb; a.sdkh = sdkh; a.sdkn = sdkn; a.sdvb = sdvb; a.sdvh = sdvh; a.sdvn = sdvn;
   a.sm_scale = sm_scale; a.causal = causal;
   if (int e = check_attn_common("attn_bwd", a)) return e;
-  if (!dout || !delta || !dq || !dk || !dv) return set_error(QFA_EINVAL, "attn_bwd: null pointer argument");
-  if (!aligned16(dout) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv))
-    return set_error(QFA_EINVAL, "attn_bwd: dout, dq, dk, dv must be 16-byte aligned");
+  if (!dout || !workspace || !dq || !dk || !dv) return set_error(QFA_EINVAL, "attn_bwd: null pointer argument");
+  if (!aligned16(dout) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv) || !aligned16(workspace))
+    return set_error(QFA_EINVAL, "attn_bwd: dout, dq, dk, dv, workspace must be 16-byte aligned");
+  const int64_t need = bwd_workspace_bytes(B, H, Nq, Nk, D);
+  if (workspace_bytes < need)
+    return set_error(QFA_EINVAL, "attn_bwd: workspace of %lld bytes is too small, need %lld (qfa_attn_bwd_workspace_bytes)",
+                     (long long)workspace_bytes, (long long)need);
   if (!strides_ok(sdob, sdoh, sdon, D, 2) || !strides_ok(sdqb, sdqh, sdqn, D, 2) ||
       !strides_ok(sdkb, sdkh, sdkn, D, 2) || !strides_ok(sdvb, sdvh, sdvn, D, 2))
     return set_error(QFA_EINVAL, "attn_bwd: strides must be positive multiples of 16 bytes, token stride >= D");
-  if (int e = launch_delta(o, dout, delta, io_dtype, B, H, Nq, D, sob, soh, son, sdob, sdoh, sdon, (hipStream_t)stream))
-    return e;
   return launch_bwd(a, (hipStream_t)stream);
 }
 

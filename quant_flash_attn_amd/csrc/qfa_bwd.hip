@@ -1,6 +1,11 @@
-// Backward kernels for gfx950: delta = rowsum(O o dO), then two MFMA kernels that recompute
+// Backward kernels for gfx950: two staging passes, then two MFMA kernels that recompute
 // P = exp(S - LSE) from the INT8 codes exactly as the forward does.
 //
+//   prep_q       per 64-query tile: delta = rowsum(O o dO) in fp32; dO^T and Qz^T = (Qc - zq)^T as
+//                16-bit tiles [d][query] in the key order the MFMA layouts want; per-query constants
+//   prep_k       per 64-key tile: Kz^T = (Kc - zk)^T likewise; per-key constants
+//                (both write into the caller's workspace; every tile is converted and transposed
+//                once instead of once per consuming workgroup)
 //   dq kernel    one workgroup = 128 queries (32 per wave), loops over 64-key tiles.
 //                S^T = Kc.Qc^T (INT8 MFMA), dP^T = V.dO^T, dS^T = P^T o (dP^T - delta),
 //                dQ^T += Kz^T.(dS^T * sk)         with Kz = (Kc - zk) held as exact 16-bit floats
@@ -73,24 +78,43 @@ int launch_delta(const void *o, const void *dout, float *delta, int io_dtype, in
 }
 
 // ------------------------------------------------------------------------------------------ shared
+constexpr int BWD_BLK = 128;   // rows owned by a workgroup
+constexpr int BWD_TILE = 64;   // rows streamed per step
+
+// Workspace layout: per (batch*head, 64-query tile) a Q-side blob, then per (batch*head, 64-key tile)
+// a K-side blob.  Transposed tiles are [D][64] 16-bit values, 128-byte rows, positions permuted.
+template <int D> struct BwdWs {
+  static constexpr int T_BYTES = D * BWD_TILE * 2;            // one transposed tile
+  static constexpr int CQ_BYTES = 5 * BWD_TILE * 4;           // digits (2 dwords/query), a, -lse*log2e, delta
+  static constexpr int CK_BYTES = 3 * BWD_TILE * 4;           // digits (2 dwords/key), key scale
+  static constexpr int Q_BLOB = 2 * T_BYTES + CQ_BYTES;       // dO^T, Qz^T, constants
+  static constexpr int K_BLOB = T_BYTES + CK_BYTES;           // Kz^T, constants
+};
+
+int64_t bwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D) {
+  const int64_t tq = (Nq + BWD_TILE - 1) / BWD_TILE, tk = (Nk + BWD_TILE - 1) / BWD_TILE;
+  const int64_t qb = D == 128 ? BwdWs<128>::Q_BLOB : BwdWs<64>::Q_BLOB;
+  const int64_t kb = D == 128 ? BwdWs<128>::K_BLOB : BwdWs<64>::K_BLOB;
+  return B * H * (tq * qb + tk * kb);
+}
+
 struct BwdArgs {
   const int8_t *qc; const float *sq; const int8_t *zq; const int32_t *rq;
   const int8_t *kc; const float *sk; const int8_t *zk; const int32_t *rk;
-  const void *v; const void *dout; const float *lse; const float *delta;
+  const void *v; const void *o; const void *dout; const float *lse;
+  unsigned char *ws_q; unsigned char *ws_k;
   void *dq; void *dk; void *dv;
   int64_t H;
   int Nq, Nk;
-  int64_t sqb, sqh, sqn, skb, skh, skn, svb, svh, svn;
+  int tiles_q, tiles_k;
+  int64_t sqb, sqh, sqn, skb, skh, skn, svb, svh, svn, sob, soh, son;
   int64_t sdob, sdoh, sdon, sdqb, sdqh, sdqn, sdkb, sdkh, sdkn, sdvb, sdvh, sdvn;
   float sm_scale, sm_scale_log2;
   int nblocks;          // query blocks (dq) or key blocks (dkdv) per (b,h)
   int total_blocks, blocks_per_xcd;
 };
 
-constexpr int BWD_BLK = 128;   // rows owned by a workgroup
-constexpr int BWD_TILE = 64;   // rows streamed per step
-
-// position of streamed row r (0..63) inside a transposed LDS tile: the order in which the 32x32
+// position of streamed row r (0..63) inside a transposed tile: the order in which the 32x32
 // accumulator layout hands out rows to a lane (two runs of 4 per 16-row MFMA k-slice)
 __device__ __forceinline__ int perm_pos4(int r4) {   // r4 = r / 4
   return 32 * (r4 / 8) + 16 * ((r4 / 4) % 2) + 8 * (r4 % 2) + 4 * ((r4 / 2) % 2);
@@ -128,25 +152,151 @@ __device__ __forceinline__ void store_16b_transposed(const u32x4 (&w)[4], unsign
     *reinterpret_cast<u32x2 *>(dst + e * stride) = o;
   }
 }
+// integer n -> (128*floor(n/128), n mod 128) resp. their negatives, as a packed pair of 16-bit floats
+template <typename T> __device__ __forceinline__ unsigned base128_pair(int n, float sign) {
+  const int hi = n >> 7, lo = n & 127;
+  return pack2<T>(sign * (float)(hi * 128), sign * (float)lo);
+}
+
+// ------------------------------------------------------------------------------------------ prep
+// One block per (b,h, 64-query tile): delta, dO^T, Qz^T and the per-query constants.
+template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_q_kernel(BwdArgs a) {
+  typedef BwdWs<D> WS;
+  __shared__ float red[D / 8][BWD_TILE];
+  const int tid = threadIdx.x;
+  const int bh = blockIdx.x / a.tiles_q, tile = blockIdx.x % a.tiles_q;
+  const int64_t b = bh / a.H, h = bh % a.H;
+  const int i0 = tile * BWD_TILE;
+  const int64_t tq0 = (int64_t)bh * a.Nq;
+  unsigned char *blob = a.ws_q + ((int64_t)bh * a.tiles_q + tile) * WS::Q_BLOB;
+  const int r4 = tid % 16, dc = tid / 16;
+  if (dc < D / 8) {
+    const int8_t *qc_bh = a.qc + b * a.sqb + h * a.sqh;
+    const T *do_bh = reinterpret_cast<const T *>(a.dout) + b * a.sdob + h * a.sdoh;
+    const T *o_bh = reinterpret_cast<const T *>(a.o) + b * a.sob + h * a.soh;
+    u32x2 creg[4];
+    u32x4 greg[4];
+    float zreg[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int i = min(i0 + 4 * r4 + r, a.Nq - 1);
+      creg[r] = *reinterpret_cast<const u32x2 *>(qc_bh + (int64_t)i * a.sqn + dc * 8);
+      greg[r] = *reinterpret_cast<const u32x4 *>(do_bh + (int64_t)i * a.sdon + dc * 8);
+      const u32x4 ow = *reinterpret_cast<const u32x4 *>(o_bh + (int64_t)i * a.son + dc * 8);
+      zreg[r] = (float)a.zq[tq0 + i];
+      float s = 0.f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        s = __builtin_fmaf(lo_to_f32<T>(ow[e]), lo_to_f32<T>(greg[r][e]), s);
+        s = __builtin_fmaf(hi_to_f32<T>(ow[e]), hi_to_f32<T>(greg[r][e]), s);
+      }
+      red[dc][4 * r4 + r] = s;
+    }
+    const int pos = perm_pos4(r4);
+    store_16b_transposed(greg, blob + (dc * 8) * (BWD_TILE * 2) + pos * 2, BWD_TILE * 2);
+    store_codes_transposed<T>(creg, zreg, blob + WS::T_BYTES + (dc * 8) * (BWD_TILE * 2) + pos * 2, BWD_TILE * 2);
+  }
+  __syncthreads();
+  if (tid < BWD_TILE) {
+    const int i = min(i0 + tid, a.Nq - 1);
+    float delta = 0.f;
+#pragma unroll
+    for (int x = 0; x < D / 8; ++x) delta += red[x][tid];
+    const int zq = (int)a.zq[tq0 + i];
+    const int c = a.rq[tq0 + i] - D * zq;
+    unsigned *cq = reinterpret_cast<unsigned *>(blob + 2 * WS::T_BYTES);
+    u32x2 dg;
+    dg[0] = pack2<T>((float)(-zq), (float)(-zq));      // k-group 0: times the two digits of rk
+    dg[1] = base128_pair<T>(c, -1.0f);                 // k-group 1: minus the digits of rq - D*zq, times zk
+    reinterpret_cast<u32x2 *>(cq)[tid] = dg;
+    reinterpret_cast<float *>(cq)[2 * BWD_TILE + tid] = a.sq[tq0 + i] * a.sm_scale_log2;
+    reinterpret_cast<float *>(cq)[3 * BWD_TILE + tid] = -a.lse[tq0 + i] * kLog2e;
+    reinterpret_cast<float *>(cq)[4 * BWD_TILE + tid] = delta;
+  }
+}
+
+// One block per (b,h, 64-key tile): Kz^T and the per-key constants.
+template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_k_kernel(BwdArgs a) {
+  typedef BwdWs<D> WS;
+  const int tid = threadIdx.x;
+  const int bh = blockIdx.x / a.tiles_k, tile = blockIdx.x % a.tiles_k;
+  const int64_t b = bh / a.H, h = bh % a.H;
+  const int j0 = tile * BWD_TILE;
+  const int64_t tk0 = (int64_t)bh * a.Nk;
+  unsigned char *blob = a.ws_k + ((int64_t)bh * a.tiles_k + tile) * WS::K_BLOB;
+  const int r4 = tid % 16, dc = tid / 16;
+  if (dc < D / 8) {
+    const int8_t *kc_bh = a.kc + b * a.skb + h * a.skh;
+    u32x2 creg[4];
+    float zreg[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int j = min(j0 + 4 * r4 + r, a.Nk - 1);
+      creg[r] = *reinterpret_cast<const u32x2 *>(kc_bh + (int64_t)j * a.skn + dc * 8);
+      zreg[r] = (float)a.zk[tk0 + j];
+    }
+    store_codes_transposed<T>(creg, zreg, blob + (dc * 8) * (BWD_TILE * 2) + perm_pos4(r4) * 2, BWD_TILE * 2);
+  }
+  if (tid < BWD_TILE) {
+    const int j = min(j0 + tid, a.Nk - 1);
+    const int zk = (int)a.zk[tk0 + j];
+    unsigned *ck = reinterpret_cast<unsigned *>(blob + WS::T_BYTES);
+    u32x2 dg;
+    dg[0] = base128_pair<T>(a.rk[tk0 + j], 1.0f);      // k-group 0: digits of rk
+    dg[1] = pack2<T>((float)zk, (float)zk);            // k-group 1: zk, zk
+    reinterpret_cast<u32x2 *>(ck)[tid] = dg;
+    reinterpret_cast<float *>(ck)[2 * BWD_TILE + tid] = a.sk[tk0 + j];
+  }
+}
 
 template <int D> struct BwdSmem {
   static constexpr int CSTR = D + 16;                // int8 code rows
   static constexpr int RSTR = 2 * D + 16;            // row-major 16-bit rows
-  static constexpr int TSTR = (BWD_TILE + 8) * 2;    // transposed 16-bit rows
+  static constexpr int TSTR = BWD_TILE * 2 + 16;     // transposed 16-bit rows
   static constexpr int C_BYTES = BWD_TILE * CSTR;
   static constexpr int R_BYTES = BWD_TILE * RSTR;
   static constexpr int T_BYTES = D * TSTR;
+};
+
+// 16-byte-chunk copy of `rows` rows of `row_bytes` bytes each, global (stride gstride) -> registers
+// -> LDS (stride lstride); CH = chunks per thread (rows*row_bytes/16/256, rounded up)
+template <int CH> struct Stage {
+  u32x4 r[CH];
+  __device__ __forceinline__ void load(const unsigned char *g, int64_t gstride, int rows, int row_bytes, int row0,
+                                       int row_max, int tid) {
+    const int cpr = row_bytes / 16;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c / cpr, col = c % cpr;
+      if (row < rows) {
+        const int rr = min(row0 + row, row_max);
+        r[i] = *reinterpret_cast<const u32x4 *>(g + (int64_t)rr * gstride + col * 16);
+      }
+    }
+  }
+  __device__ __forceinline__ void store(unsigned char *l, int lstride, int rows, int row_bytes, int tid) const {
+    const int cpr = row_bytes / 16;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c / cpr, col = c % cpr;
+      if (row < rows) *reinterpret_cast<u32x4 *>(l + row * lstride + col * 16) = r[i];
+    }
+  }
 };
 
 // ------------------------------------------------------------------------------------------ dQ
 template <typename T, int D, bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdArgs a) {
   typedef BwdSmem<D> SM;
+  typedef BwdWs<D> WS;
   constexpr int KS = D / 32, DB = D / 32, KD = D / 16;
-  constexpr int KCH = (BWD_TILE * D / 16) / 256;
-  constexpr int VCH = (BWD_TILE * D / 8) / 256;
+  constexpr int KCH = (BWD_TILE * D / 16 + 255) / 256;
+  constexpr int VCH = (BWD_TILE * 2 * D / 16 + 255) / 256;
+  constexpr int TCH = (D * BWD_TILE * 2 / 16 + 255) / 256;
   constexpr int OFF_V = SM::C_BYTES, OFF_T = OFF_V + SM::R_BYTES, OFF_C = OFF_T + SM::T_BYTES;
-  __shared__ __attribute__((aligned(16))) unsigned char smem[OFF_C + 3 * BWD_TILE * 4];
+  __shared__ __attribute__((aligned(16))) unsigned char smem[OFF_C + WS::CK_BYTES];
 
   const int L = blockIdx.x;
   const int vid = (L % 8) * a.blocks_per_xcd + (L / 8);
@@ -159,11 +309,13 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdArgs a) {
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, lr = lane % 32, g = lane / 32;
 
   const int8_t *qc_bh = a.qc + b * a.sqb + h * a.sqh;
-  const int8_t *kc_bh = a.kc + b * a.skb + h * a.skh;
-  const T *v_bh = reinterpret_cast<const T *>(a.v) + b * a.svb + h * a.svh;
+  const unsigned char *kc_bh = reinterpret_cast<const unsigned char *>(a.kc + b * a.skb + h * a.skh);
+  const unsigned char *v_bh = reinterpret_cast<const unsigned char *>(reinterpret_cast<const T *>(a.v) + b * a.svb + h * a.svh);
   const T *do_bh = reinterpret_cast<const T *>(a.dout) + b * a.sdob + h * a.sdoh;
   T *dq_bh = reinterpret_cast<T *>(a.dq) + b * a.sdqb + h * a.sdqh;
-  const int64_t tq0 = (int64_t)bh * a.Nq, tk0 = (int64_t)bh * a.Nk;
+  const int64_t tq0 = (int64_t)bh * a.Nq;
+  const unsigned char *wsk_bh = a.ws_k + (int64_t)bh * a.tiles_k * WS::K_BLOB;
+  const unsigned char *wsq_bh = a.ws_q + (int64_t)bh * a.tiles_q * WS::Q_BLOB;
 
   const int qi = m0 + wave * 32 + lr;
   const int qi_c = qi < a.Nq ? qi : a.Nq - 1;
@@ -175,75 +327,37 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdArgs a) {
 #pragma unroll
   for (int kd = 0; kd < KD; ++kd)
     dof[kd] = *reinterpret_cast<const u32x4 *>(do_bh + (int64_t)qi_c * a.sdon + kd * 16 + g * 8);
-  const float zqf = (float)a.zq[tq0 + qi_c];
-  const float a_i = a.sq[tq0 + qi_c] * a.sm_scale_log2;
-  const float nzq = -zqf;
-  const float nc = -((float)a.rq[tq0 + qi_c] - (float)D * zqf);
-  const float nlse2 = -a.lse[tq0 + qi_c] * kLog2e;
-  const float delta_i = a.delta[tq0 + qi_c];
+  // per-query constants prepared by prep_q: correction digits, a = sq*sm*log2e, -lse*log2e, delta
+  const unsigned *cq = reinterpret_cast<const unsigned *>(wsq_bh + (int64_t)(qi_c / BWD_TILE) * WS::Q_BLOB + 2 * WS::T_BYTES);
+  const int ql = qi_c % BWD_TILE;
+  u32x4 corr_q = {cq[2 * ql + g], 0u, 0u, 0u};
+  const float a_i = __builtin_bit_cast(float, cq[2 * BWD_TILE + ql]);
+  const float nlse2 = __builtin_bit_cast(float, cq[3 * BWD_TILE + ql]);
+  const float delta_i = __builtin_bit_cast(float, cq[4 * BWD_TILE + ql]);
+  (void)tq0;
   const int q_first = m0 + wave * 32, q_last = q_first + 31;
 
   int kv_end = a.Nk;
   if (CAUSAL) kv_end = min(a.Nk, m0 + BWD_BLK);
   const int ntiles = (kv_end + BWD_TILE - 1) / BWD_TILE;
 
-  const int t_r4 = tid % 16, t_dc = tid / 16;
-  const bool t_active = t_dc < D / 8;
-  const int t_pos = perm_pos4(t_r4);
-
-  u32x4 kreg[KCH], vreg[VCH];
-  u32x2 creg[4];
-  float zreg[4];
-  float cst[3];
-
+  Stage<KCH> st_k;
+  Stage<VCH> st_v;
+  Stage<TCH> st_t;
+  u32x4 st_c;
   auto load_tile = [&](int t) {
     const int j0 = t * BWD_TILE;
-#pragma unroll
-    for (int i = 0; i < KCH; ++i) {
-      const int c = tid + 256 * i, row = c / (D / 16), col = c % (D / 16);
-      const int j = min(j0 + row, a.Nk - 1);
-      kreg[i] = *reinterpret_cast<const u32x4 *>(kc_bh + (int64_t)j * a.skn + col * 16);
-    }
-#pragma unroll
-    for (int i = 0; i < VCH; ++i) {
-      const int c = tid + 256 * i, row = c / (D / 8), col = c % (D / 8);
-      const int j = min(j0 + row, a.Nk - 1);
-      vreg[i] = *reinterpret_cast<const u32x4 *>(v_bh + (int64_t)j * a.svn + col * 8);
-    }
-    if (t_active) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int j = min(j0 + 4 * t_r4 + r, a.Nk - 1);
-        creg[r] = *reinterpret_cast<const u32x2 *>(kc_bh + (int64_t)j * a.skn + t_dc * 8);
-        zreg[r] = (float)a.zk[tk0 + j];
-      }
-    }
-    if (tid < BWD_TILE) {
-      const int j = min(j0 + tid, a.Nk - 1);
-      cst[0] = a.sk[tk0 + j];
-      cst[1] = (float)a.rk[tk0 + j];
-      cst[2] = (float)a.zk[tk0 + j];
-    }
+    const unsigned char *blob = wsk_bh + (int64_t)t * WS::K_BLOB;
+    st_k.load(kc_bh, a.skn, BWD_TILE, D, j0, a.Nk - 1, tid);
+    st_v.load(v_bh, a.svn * 2, BWD_TILE, 2 * D, j0, a.Nk - 1, tid);
+    st_t.load(blob, BWD_TILE * 2, D, BWD_TILE * 2, 0, D - 1, tid);
+    if (tid < WS::CK_BYTES / 16) st_c = *reinterpret_cast<const u32x4 *>(blob + WS::T_BYTES + tid * 16);
   };
   auto store_tile = [&]() {
-#pragma unroll
-    for (int i = 0; i < KCH; ++i) {
-      const int c = tid + 256 * i, row = c / (D / 16), col = c % (D / 16);
-      *reinterpret_cast<u32x4 *>(smem + row * SM::CSTR + col * 16) = kreg[i];
-    }
-#pragma unroll
-    for (int i = 0; i < VCH; ++i) {
-      const int c = tid + 256 * i, row = c / (D / 8), col = c % (D / 8);
-      *reinterpret_cast<u32x4 *>(smem + OFF_V + row * SM::RSTR + col * 16) = vreg[i];
-    }
-    if (t_active)
-      store_codes_transposed<T>(creg, zreg, smem + OFF_T + (t_dc * 8) * SM::TSTR + t_pos * 2, SM::TSTR);
-    if (tid < BWD_TILE) {
-      float *cs = reinterpret_cast<float *>(smem + OFF_C);
-      cs[tid] = cst[0];
-      cs[BWD_TILE + tid] = cst[1];
-      cs[2 * BWD_TILE + tid] = cst[2];
-    }
+    st_k.store(smem, SM::CSTR, BWD_TILE, D, tid);
+    st_v.store(smem + OFF_V, SM::RSTR, BWD_TILE, 2 * D, tid);
+    st_t.store(smem + OFF_T, SM::TSTR, D, BWD_TILE * 2, tid);
+    if (tid < WS::CK_BYTES / 16) *reinterpret_cast<u32x4 *>(smem + OFF_C + tid * 16) = st_c;
   };
 
   f32x16 dqacc[DB];
@@ -258,7 +372,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdArgs a) {
     __syncthreads();
     if (t + 1 < ntiles) load_tile(t + 1);
 
-    const float *cs = reinterpret_cast<const float *>(smem + OFF_C);
+    const unsigned *dgp = reinterpret_cast<const unsigned *>(smem + OFF_C);
+    const float *skp = reinterpret_cast<const float *>(smem + OFF_C) + 2 * BWD_TILE;
     const int j0 = t * BWD_TILE;
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
@@ -279,21 +394,21 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdArgs a) {
         const u32x4 vf = *reinterpret_cast<const u32x4 *>(smem + OFF_V + (32 * nb + lr) * SM::RSTR + kd * 32 + g * 16);
         dp = mfma_16b<T>(vf, dof[kd], dp);
       }
+      f32x16 f;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) f[v] = (float)acc[v];
+      const u32x4 corr_k = {dgp[2 * (32 * nb + lr) + g], 0u, 0u, 0u};
+      f = mfma_16b<T>(corr_k, corr_q, f);
       const bool need_mask = (CAUSAL && jb + 31 > q_first) || (jb + 32 > a.Nk);
       float ds[16];
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa) {
         const int jl = 32 * nb + 8 * aa + 4 * g;
-        const f32x4 sk4 = *reinterpret_cast<const f32x4 *>(cs + jl);
-        const f32x4 rk4 = *reinterpret_cast<const f32x4 *>(cs + BWD_TILE + jl);
-        const f32x4 zk4 = *reinterpret_cast<const f32x4 *>(cs + 2 * BWD_TILE + jl);
+        const f32x4 sk4 = *reinterpret_cast<const f32x4 *>(skp + jl);
 #pragma unroll
         for (int bb = 0; bb < 4; ++bb) {
           const int v = 4 * aa + bb;
-          float f = (float)acc[v];
-          f = __builtin_fmaf(nzq, rk4[bb], f);
-          f = __builtin_fmaf(nc, zk4[bb], f);
-          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, f * sk4[bb], nlse2));
+          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, f[v] * sk4[bb], nlse2));
           if (need_mask) {
             const int j = j0 + jl + bb;
             if ((CAUSAL && j > qi) || j >= a.Nk) p = 0.f;
@@ -335,10 +450,14 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdArgs a) {
 template <typename T, int D, bool CAUSAL>
 __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
   typedef BwdSmem<D> SM;
+  typedef BwdWs<D> WS;
   constexpr int KS = D / 32, DB = D / 32, KD = D / 16;
+  constexpr int QCH = (BWD_TILE * D / 16 + 255) / 256;
+  constexpr int GCH = (BWD_TILE * 2 * D / 16 + 255) / 256;
+  constexpr int TCH = (D * BWD_TILE * 2 / 16 + 255) / 256;
   constexpr int OFF_DO = SM::C_BYTES, OFF_DOT = OFF_DO + SM::R_BYTES, OFF_QT = OFF_DOT + SM::T_BYTES,
-                OFF_C = OFF_QT + SM::T_BYTES;
-  __shared__ __attribute__((aligned(16))) unsigned char smem[OFF_C + 5 * BWD_TILE * 4];
+                OFF_C = OFF_QT + SM::T_BYTES, BUF = OFF_C + WS::CQ_BYTES;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF];
 
   const int L = blockIdx.x;
   const int vid = (L % 8) * a.blocks_per_xcd + (L / 8);
@@ -349,13 +468,14 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
   const int n0 = nbk * BWD_BLK;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, lr = lane % 32, g = lane / 32;
 
-  const int8_t *qc_bh = a.qc + b * a.sqb + h * a.sqh;
+  const unsigned char *qc_bh = reinterpret_cast<const unsigned char *>(a.qc + b * a.sqb + h * a.sqh);
   const int8_t *kc_bh = a.kc + b * a.skb + h * a.skh;
   const T *v_bh = reinterpret_cast<const T *>(a.v) + b * a.svb + h * a.svh;
-  const T *do_bh = reinterpret_cast<const T *>(a.dout) + b * a.sdob + h * a.sdoh;
+  const unsigned char *do_bh = reinterpret_cast<const unsigned char *>(reinterpret_cast<const T *>(a.dout) + b * a.sdob + h * a.sdoh);
   T *dk_bh = reinterpret_cast<T *>(a.dk) + b * a.sdkb + h * a.sdkh;
   T *dv_bh = reinterpret_cast<T *>(a.dv) + b * a.sdvb + h * a.sdvh;
-  const int64_t tq0 = (int64_t)bh * a.Nq, tk0 = (int64_t)bh * a.Nk;
+  const unsigned char *wsk_bh = a.ws_k + (int64_t)bh * a.tiles_k * WS::K_BLOB;
+  const unsigned char *wsq_bh = a.ws_q + (int64_t)bh * a.tiles_q * WS::Q_BLOB;
 
   // ---- this lane's key
   const int kj = n0 + wave * 32 + lr;
@@ -368,60 +488,35 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
 #pragma unroll
   for (int kd = 0; kd < KD; ++kd)
     vf[kd] = *reinterpret_cast<const u32x4 *>(v_bh + (int64_t)kj_c * a.svn + kd * 16 + g * 8);
-  const float zkf = (float)a.zk[tk0 + kj_c];
-  const float sk_j = a.sk[tk0 + kj_c];
-  const float nzk = -zkf;
-  const float nck = -((float)a.rk[tk0 + kj_c] - (float)D * zkf);
+  const unsigned *ck = reinterpret_cast<const unsigned *>(wsk_bh + (int64_t)(kj_c / BWD_TILE) * WS::K_BLOB + WS::T_BYTES);
+  const int kl = kj_c % BWD_TILE;
+  const u32x4 corr_k = {ck[2 * kl + g], 0u, 0u, 0u};
+  const float sk_j = __builtin_bit_cast(float, ck[2 * BWD_TILE + kl]);
   const int k_first = n0 + wave * 32, k_last = k_first + 31;
 
   const int it0 = CAUSAL ? n0 / BWD_TILE : 0;
-  const int ntiles = (a.Nq + BWD_TILE - 1) / BWD_TILE;
+  const int ntiles = a.tiles_q;
 
-  const int t_r4 = tid % 16, t_dc = tid / 16;
-  const bool t_active = t_dc < D / 8;
-  const int t_pos = perm_pos4(t_r4);
-
-  u32x2 creg[4];
-  u32x4 greg[4];
-  float zreg[4];
-  float cst[5];
-
+  Stage<QCH> st_q;
+  Stage<GCH> st_g;
+  Stage<TCH> st_gt, st_qt;
+  u32x4 st_c;
   auto load_tile = [&](int t) {
     const int i0 = t * BWD_TILE;
-    if (t_active) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int i = min(i0 + 4 * t_r4 + r, a.Nq - 1);
-        creg[r] = *reinterpret_cast<const u32x2 *>(qc_bh + (int64_t)i * a.sqn + t_dc * 8);
-        greg[r] = *reinterpret_cast<const u32x4 *>(do_bh + (int64_t)i * a.sdon + t_dc * 8);
-        zreg[r] = (float)a.zq[tq0 + i];
-      }
-    }
-    if (tid < BWD_TILE) {
-      const int i = min(i0 + tid, a.Nq - 1);
-      const float zq = (float)a.zq[tq0 + i];
-      cst[0] = (float)a.rq[tq0 + i];
-      cst[1] = zq;
-      cst[2] = a.sq[tq0 + i] * a.sm_scale_log2;
-      cst[3] = -a.lse[tq0 + i] * kLog2e;
-      cst[4] = a.delta[tq0 + i];
-    }
+    const unsigned char *blob = wsq_bh + (int64_t)t * WS::Q_BLOB;
+    st_q.load(qc_bh, a.sqn, BWD_TILE, D, i0, a.Nq - 1, tid);
+    st_g.load(do_bh, a.sdon * 2, BWD_TILE, 2 * D, i0, a.Nq - 1, tid);
+    st_gt.load(blob, BWD_TILE * 2, D, BWD_TILE * 2, 0, D - 1, tid);
+    st_qt.load(blob + WS::T_BYTES, BWD_TILE * 2, D, BWD_TILE * 2, 0, D - 1, tid);
+    if (tid < WS::CQ_BYTES / 16) st_c = *reinterpret_cast<const u32x4 *>(blob + 2 * WS::T_BYTES + tid * 16);
   };
-  auto store_tile = [&]() {
-    if (t_active) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        *reinterpret_cast<u32x2 *>(smem + (4 * t_r4 + r) * SM::CSTR + t_dc * 8) = creg[r];
-        *reinterpret_cast<u32x4 *>(smem + OFF_DO + (4 * t_r4 + r) * SM::RSTR + t_dc * 16) = greg[r];
-      }
-      store_16b_transposed(greg, smem + OFF_DOT + (t_dc * 8) * SM::TSTR + t_pos * 2, SM::TSTR);
-      store_codes_transposed<T>(creg, zreg, smem + OFF_QT + (t_dc * 8) * SM::TSTR + t_pos * 2, SM::TSTR);
-    }
-    if (tid < BWD_TILE) {
-      float *cs = reinterpret_cast<float *>(smem + OFF_C);
-#pragma unroll
-      for (int x = 0; x < 5; ++x) cs[x * BWD_TILE + tid] = cst[x];
-    }
+  auto store_tile = [&](int buf) {
+    unsigned char *base = smem + buf * BUF;
+    st_q.store(base, SM::CSTR, BWD_TILE, D, tid);
+    st_g.store(base + OFF_DO, SM::RSTR, BWD_TILE, 2 * D, tid);
+    st_gt.store(base + OFF_DOT, SM::TSTR, D, BWD_TILE * 2, tid);
+    st_qt.store(base + OFF_QT, SM::TSTR, D, BWD_TILE * 2, tid);
+    if (tid < WS::CQ_BYTES / 16) *reinterpret_cast<u32x4 *>(base + OFF_C + tid * 16) = st_c;
   };
 
   f32x16 dkacc[DB], dvacc[DB];
@@ -430,13 +525,17 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) { dkacc[db][v] = 0.f; dvacc[db][v] = 0.f; }
 
-  if (it0 < ntiles) load_tile(it0);
+  if (it0 < ntiles) {
+    load_tile(it0);
+    store_tile(it0 & 1);
+  }
+  __syncthreads();
   for (int t = it0; t < ntiles; ++t) {
-    store_tile();
-    __syncthreads();
     if (t + 1 < ntiles) load_tile(t + 1);
 
-    const float *cs = reinterpret_cast<const float *>(smem + OFF_C);
+    const unsigned char *base = smem + (t & 1) * BUF;
+    const unsigned *dgp = reinterpret_cast<const unsigned *>(base + OFF_C);
+    const float *cs = reinterpret_cast<const float *>(base + OFF_C);
     const int i0 = t * BWD_TILE;
 #pragma unroll
     for (int mbk = 0; mbk < 2; ++mbk) {
@@ -449,31 +548,31 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
       for (int v = 0; v < 16; ++v) { acc[v] = 0; dp[v] = 0.f; }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const i32x4 qfr = *reinterpret_cast<const i32x4 *>(smem + (32 * mbk + lr) * SM::CSTR + ks * 32 + g * 16);
+        const i32x4 qfr = *reinterpret_cast<const i32x4 *>(base + (32 * mbk + lr) * SM::CSTR + ks * 32 + g * 16);
         acc = mfma_i8(qfr, kf[ks], acc);
       }
 #pragma unroll
       for (int kd = 0; kd < KD; ++kd) {
-        const u32x4 gf = *reinterpret_cast<const u32x4 *>(smem + OFF_DO + (32 * mbk + lr) * SM::RSTR + kd * 32 + g * 16);
+        const u32x4 gf = *reinterpret_cast<const u32x4 *>(base + OFF_DO + (32 * mbk + lr) * SM::RSTR + kd * 32 + g * 16);
         dp = mfma_16b<T>(gf, vf[kd], dp);
       }
+      f32x16 f;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) f[v] = (float)acc[v];
+      const u32x4 corr_q = {dgp[2 * (32 * mbk + lr) + g], 0u, 0u, 0u};
+      f = mfma_16b<T>(corr_q, corr_k, f);
       const bool need_mask = (CAUSAL && ib < k_last) || (ib + 32 > a.Nq) || (k_last >= a.Nk);
       float pp[16], ds[16];
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa) {
         const int il = 32 * mbk + 8 * aa + 4 * g;
-        const f32x4 rq4 = *reinterpret_cast<const f32x4 *>(cs + il);
-        const f32x4 zq4 = *reinterpret_cast<const f32x4 *>(cs + BWD_TILE + il);
         const f32x4 a4 = *reinterpret_cast<const f32x4 *>(cs + 2 * BWD_TILE + il);
         const f32x4 nl4 = *reinterpret_cast<const f32x4 *>(cs + 3 * BWD_TILE + il);
         const f32x4 dl4 = *reinterpret_cast<const f32x4 *>(cs + 4 * BWD_TILE + il);
 #pragma unroll
         for (int bb = 0; bb < 4; ++bb) {
           const int v = 4 * aa + bb;
-          float f = (float)acc[v];
-          f = __builtin_fmaf(nzk, rq4[bb], f);
-          f = __builtin_fmaf(nck, zq4[bb], f);
-          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a4[bb], f * sk_j, nl4[bb]));
+          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a4[bb], f[v] * sk_j, nl4[bb]));
           if (need_mask) {
             const int i = i0 + il + bb;
             if ((CAUSAL && kj > i) || i >= a.Nq || kj >= a.Nk) p = 0.f;
@@ -493,13 +592,14 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
           const int off = (32 * db + lr) * SM::TSTR + (32 * mbk + 16 * hh + 8 * g) * 2;
-          const u32x4 gtf = *reinterpret_cast<const u32x4 *>(smem + OFF_DOT + off);
+          const u32x4 gtf = *reinterpret_cast<const u32x4 *>(base + OFF_DOT + off);
           dvacc[db] = mfma_16b<T>(gtf, pf, dvacc[db]);
-          const u32x4 qtf = *reinterpret_cast<const u32x4 *>(smem + OFF_QT + off);
+          const u32x4 qtf = *reinterpret_cast<const u32x4 *>(base + OFF_QT + off);
           dkacc[db] = mfma_16b<T>(qtf, dsf, dkacc[db]);
         }
       }
     }
+    if (t + 1 < ntiles) store_tile((t + 1) & 1);
     __syncthreads();
   }
 
@@ -522,20 +622,34 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
 }
 
 template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStream_t st) {
+  typedef BwdWs<D> WS;
   BwdArgs a;
   a.qc = x.qc; a.sq = x.sq; a.zq = x.zq; a.rq = x.rq; a.kc = x.kc; a.sk = x.sk; a.zk = x.zk; a.rk = x.rk;
-  a.v = x.v; a.dout = x.dout; a.lse = x.lse; a.delta = x.delta; a.dq = x.dq; a.dk = x.dk; a.dv = x.dv;
+  a.v = x.v; a.o = x.o; a.dout = x.dout; a.lse = x.lse; a.dq = x.dq; a.dk = x.dk; a.dv = x.dv;
   a.H = x.H; a.Nq = (int)x.Nq; a.Nk = (int)x.Nk;
+  a.tiles_q = (int)((x.Nq + BWD_TILE - 1) / BWD_TILE);
+  a.tiles_k = (int)((x.Nk + BWD_TILE - 1) / BWD_TILE);
+  a.ws_q = reinterpret_cast<unsigned char *>(x.workspace);
+  a.ws_k = a.ws_q + x.B * x.H * (int64_t)a.tiles_q * WS::Q_BLOB;
   a.sqb = x.sqb; a.sqh = x.sqh; a.sqn = x.sqn; a.skb = x.skb; a.skh = x.skh; a.skn = x.skn;
-  a.svb = x.svb; a.svh = x.svh; a.svn = x.svn;
+  a.svb = x.svb; a.svh = x.svh; a.svn = x.svn; a.sob = x.sob; a.soh = x.soh; a.son = x.son;
   a.sdob = x.sdob; a.sdoh = x.sdoh; a.sdon = x.sdon; a.sdqb = x.sdqb; a.sdqh = x.sdqh; a.sdqn = x.sdqn;
   a.sdkb = x.sdkb; a.sdkh = x.sdkh; a.sdkn = x.sdkn; a.sdvb = x.sdvb; a.sdvh = x.sdvh; a.sdvn = x.sdvn;
   a.sm_scale = x.sm_scale; a.sm_scale_log2 = x.sm_scale * kLog2e;
+  a.nblocks = 0; a.total_blocks = 0; a.blocks_per_xcd = 0;
   const dim3 block(256);
+  const int64_t BH = x.B * x.H;
+  if (BH * a.tiles_q > 0x7fffffffLL || BH * a.tiles_k > 0x7fffffffLL)
+    return set_error(QFA_EUNSUPPORTED, "attn_bwd: too many tiles for one launch");
+  // staging passes
+  bwd_prep_q_kernel<T, D><<<dim3((unsigned)(BH * a.tiles_q)), block, 0, st>>>(a);
+  if (int e = check_launch("qfa_attn_bwd (prep q)")) return e;
+  bwd_prep_k_kernel<T, D><<<dim3((unsigned)(BH * a.tiles_k)), block, 0, st>>>(a);
+  if (int e = check_launch("qfa_attn_bwd (prep k)")) return e;
   // dK, dV
   {
     a.nblocks = (int)((x.Nk + BWD_BLK - 1) / BWD_BLK);
-    const int64_t total = (int64_t)a.nblocks * x.B * x.H;
+    const int64_t total = (int64_t)a.nblocks * BH;
     if (total > 0x3fffffffLL) return set_error(QFA_EUNSUPPORTED, "attn_bwd: too many key blocks for one launch");
     a.total_blocks = (int)total;
     a.blocks_per_xcd = (a.total_blocks + 7) / 8;
@@ -547,7 +661,7 @@ template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStre
   // dQ
   {
     a.nblocks = (int)((x.Nq + BWD_BLK - 1) / BWD_BLK);
-    const int64_t total = (int64_t)a.nblocks * x.B * x.H;
+    const int64_t total = (int64_t)a.nblocks * BH;
     if (total > 0x3fffffffLL) return set_error(QFA_EUNSUPPORTED, "attn_bwd: too many query blocks for one launch");
     a.total_blocks = (int)total;
     a.blocks_per_xcd = (a.total_blocks + 7) / 8;

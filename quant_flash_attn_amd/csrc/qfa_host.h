@@ -25,7 +25,7 @@ struct AttnArgs {
   const int8_t *qc; const float *sq; const int8_t *zq; const int32_t *rq;
   const int8_t *kc; const float *sk; const int8_t *zk; const int32_t *rk;
   const void *v; void *o; float *lse;
-  const void *dout; float *delta; void *dq; void *dk; void *dv;   // backward only
+  const void *dout; void *workspace; void *dq; void *dk; void *dv;   // backward only
   int64_t B, H, Nq, Nk;
   int64_t sqb, sqh, sqn, skb, skh, skn, svb, svh, svn, sob, soh, son;
   int64_t sdob, sdoh, sdon, sdqb, sdqh, sdqn, sdkb, sdkh, sdkn, sdvb, sdvh, sdvn;
@@ -39,5 +39,6 @@ int launch_fwd(const AttnArgs &a, hipStream_t st);
 int launch_delta(const void *o, const void *dout, float *delta, int io_dtype, int64_t B, int64_t H, int64_t N, int D,
                  int64_t sob, int64_t soh, int64_t son, int64_t sdb, int64_t sdh, int64_t sdn, hipStream_t st);
 int launch_bwd(const AttnArgs &a, hipStream_t st);
+int64_t bwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D);
 
 }  // namespace qfa

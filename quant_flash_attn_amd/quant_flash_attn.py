@@ -97,7 +97,10 @@ def attn_bwd_quantized(qq: QuantizedTokens, kq: QuantizedTokens, v: torch.Tensor
     _lib.require_gpu(qc, kc, v, o, do, lse)
     v, o, do = _rows16(v), _rows16(o), _rows16(do)
     lse = _flat(lse, torch.float32, B * H * Nq, "lse")
-    delta = torch.empty((B, H, Nq), dtype=torch.float32, device=v.device)
+    ws_bytes = _lib.lib().qfa_attn_bwd_workspace_bytes(B, H, Nq, Nk, D)
+    if ws_bytes <= 0:
+        raise ValueError(f"unsupported backward shape B={B} H={H} Nq={Nq} Nk={Nk} D={D}")
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=v.device)
     dq = torch.empty((B, H, Nq, D), dtype=v.dtype, device=v.device)
     dk = torch.empty((B, H, Nk, D), dtype=v.dtype, device=v.device)
     dv = torch.empty((B, H, Nk, D), dtype=v.dtype, device=v.device)
@@ -106,7 +109,7 @@ def attn_bwd_quantized(qq: QuantizedTokens, kq: QuantizedTokens, v: torch.Tensor
         code = _lib.lib().qfa_attn_bwd(
             qc.data_ptr(), sq.data_ptr(), zq.data_ptr(), rq.data_ptr(),
             kc.data_ptr(), sk.data_ptr(), zk.data_ptr(), rk.data_ptr(),
-            v.data_ptr(), o.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            v.data_ptr(), o.data_ptr(), do.data_ptr(), lse.data_ptr(), workspace.data_ptr(), ws_bytes,
             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), _lib.DTYPE_CODE[v.dtype],
             B, H, Nq, Nk, D, *s(qc), *s(kc), *s(v), *s(o), *s(do), *s(dq), *s(dk), *s(dv),
             float(sm_scale), int(bool(causal)), _lib.stream_of(v))
