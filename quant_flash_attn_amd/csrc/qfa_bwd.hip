@@ -19,6 +19,8 @@
 // dQ is produced by its own kernel instead of atomics, so results are deterministic.
 // (Kc - zk) and (Qc - zq) are integers in [-255, 255]: exact in bf16 and fp16, so the scales are
 // folded into dS in fp32 and dequantization adds no rounding error.
+#include <type_traits>
+
 #include "qfa_device.h"
 #include "qfa_host.h"
 
@@ -249,54 +251,20 @@ template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_k_k
   }
 }
 
-template <int D> struct BwdSmem {
-  static constexpr int CSTR = D + 16;                // int8 code rows
-  static constexpr int RSTR = 2 * D + 16;            // row-major 16-bit rows
-  static constexpr int TSTR = BWD_TILE * 2 + 16;     // transposed 16-bit rows
-  static constexpr int C_BYTES = BWD_TILE * CSTR;
-  static constexpr int R_BYTES = BWD_TILE * RSTR;
-  static constexpr int T_BYTES = D * TSTR;
-};
-
-// 16-byte-chunk copy of `rows` rows of `row_bytes` bytes each, global (stride gstride) -> registers
-// -> LDS (stride lstride); CH = chunks per thread (rows*row_bytes/16/256, rounded up)
-template <int CH> struct Stage {
-  u32x4 r[CH];
-  __device__ __forceinline__ void load(const unsigned char *g, int64_t gstride, int rows, int row_bytes, int row0,
-                                       int row_max, int tid) {
-    const int cpr = row_bytes / 16;
-#pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      const int c = tid + 256 * i;
-      const int row = c / cpr, col = c % cpr;
-      if (row < rows) {
-        const int rr = min(row0 + row, row_max);
-        r[i] = *reinterpret_cast<const u32x4 *>(g + (int64_t)rr * gstride + col * 16);
-      }
-    }
-  }
-  __device__ __forceinline__ void store(unsigned char *l, int lstride, int rows, int row_bytes, int tid) const {
-    const int cpr = row_bytes / 16;
-#pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      const int c = tid + 256 * i;
-      const int row = c / cpr, col = c % cpr;
-      if (row < rows) *reinterpret_cast<u32x4 *>(l + row * lstride + col * 16) = r[i];
-    }
-  }
-};
-
 // ------------------------------------------------------------------------------------------ dQ
+constexpr int DQ_THREADS = 512;            // 8 waves = 256 queries per workgroup
+constexpr int DQ_BLK = 32 * (DQ_THREADS / 64);
+
 template <typename T, int D, bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdArgs a) {
-  typedef BwdSmem<D> SM;
+__global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(BwdArgs a) {
   typedef BwdWs<D> WS;
+  typedef Swz<D> SK;            // K code rows
+  typedef Swz<2 * D> SV;        // V rows
+  typedef Swz<BWD_TILE * 2> ST; // transposed rows
   constexpr int KS = D / 32, DB = D / 32, KD = D / 16;
-  constexpr int KCH = (BWD_TILE * D / 16 + 255) / 256;
-  constexpr int VCH = (BWD_TILE * 2 * D / 16 + 255) / 256;
-  constexpr int TCH = (D * BWD_TILE * 2 / 16 + 255) / 256;
-  constexpr int OFF_V = SM::C_BYTES, OFF_T = OFF_V + SM::R_BYTES, OFF_C = OFF_T + SM::T_BYTES;
-  __shared__ __attribute__((aligned(16))) unsigned char smem[OFF_C + WS::CK_BYTES];
+  constexpr int K_BYTES = BWD_TILE * D, V_BYTES = BWD_TILE * 2 * D, T_BYTES = WS::T_BYTES;
+  constexpr int OFF_V = K_BYTES, OFF_T = OFF_V + V_BYTES, OFF_C = OFF_T + T_BYTES, BUF = OFF_C + WS::CK_BYTES;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF];
 
   const int L = blockIdx.x;
   const int vid = (L % 8) * a.blocks_per_xcd + (L / 8);
@@ -305,7 +273,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdArgs a) {
   int mb = vid % a.nblocks;
   if (CAUSAL) mb = a.nblocks - 1 - mb;
   const int64_t b = bh / a.H, h = bh % a.H;
-  const int m0 = mb * BWD_BLK;
+  const int m0 = mb * DQ_BLK;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, lr = lane % 32, g = lane / 32;
 
   const int8_t *qc_bh = a.qc + b * a.sqb + h * a.sqh;
@@ -313,7 +281,6 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdArgs a) {
   const unsigned char *v_bh = reinterpret_cast<const unsigned char *>(reinterpret_cast<const T *>(a.v) + b * a.svb + h * a.svh);
   const T *do_bh = reinterpret_cast<const T *>(a.dout) + b * a.sdob + h * a.sdoh;
   T *dq_bh = reinterpret_cast<T *>(a.dq) + b * a.sdqb + h * a.sdqh;
-  const int64_t tq0 = (int64_t)bh * a.Nq;
   const unsigned char *wsk_bh = a.ws_k + (int64_t)bh * a.tiles_k * WS::K_BLOB;
   const unsigned char *wsq_bh = a.ws_q + (int64_t)bh * a.tiles_q * WS::Q_BLOB;
 
@@ -330,34 +297,23 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdArgs a) {
   // per-query constants prepared by prep_q: correction digits, a = sq*sm*log2e, -lse*log2e, delta
   const unsigned *cq = reinterpret_cast<const unsigned *>(wsq_bh + (int64_t)(qi_c / BWD_TILE) * WS::Q_BLOB + 2 * WS::T_BYTES);
   const int ql = qi_c % BWD_TILE;
-  u32x4 corr_q = {cq[2 * ql + g], 0u, 0u, 0u};
+  const u32x4 corr_q = {cq[2 * ql + g], 0u, 0u, 0u};
   const float a_i = __builtin_bit_cast(float, cq[2 * BWD_TILE + ql]);
   const float nlse2 = __builtin_bit_cast(float, cq[3 * BWD_TILE + ql]);
   const float delta_i = __builtin_bit_cast(float, cq[4 * BWD_TILE + ql]);
-  (void)tq0;
   const int q_first = m0 + wave * 32, q_last = q_first + 31;
 
   int kv_end = a.Nk;
-  if (CAUSAL) kv_end = min(a.Nk, m0 + BWD_BLK);
+  if (CAUSAL) kv_end = min(a.Nk, m0 + DQ_BLK);
   const int ntiles = (kv_end + BWD_TILE - 1) / BWD_TILE;
 
-  Stage<KCH> st_k;
-  Stage<VCH> st_v;
-  Stage<TCH> st_t;
-  u32x4 st_c;
   auto load_tile = [&](int t) {
-    const int j0 = t * BWD_TILE;
+    unsigned char *base = smem + (t & 1) * BUF;
     const unsigned char *blob = wsk_bh + (int64_t)t * WS::K_BLOB;
-    st_k.load(kc_bh, a.skn, BWD_TILE, D, j0, a.Nk - 1, tid);
-    st_v.load(v_bh, a.svn * 2, BWD_TILE, 2 * D, j0, a.Nk - 1, tid);
-    st_t.load(blob, BWD_TILE * 2, D, BWD_TILE * 2, 0, D - 1, tid);
-    if (tid < WS::CK_BYTES / 16) st_c = *reinterpret_cast<const u32x4 *>(blob + WS::T_BYTES + tid * 16);
-  };
-  auto store_tile = [&]() {
-    st_k.store(smem, SM::CSTR, BWD_TILE, D, tid);
-    st_v.store(smem + OFF_V, SM::RSTR, BWD_TILE, 2 * D, tid);
-    st_t.store(smem + OFF_T, SM::TSTR, D, BWD_TILE * 2, tid);
-    if (tid < WS::CK_BYTES / 16) *reinterpret_cast<u32x4 *>(smem + OFF_C + tid * 16) = st_c;
+    dma_rows<D, BWD_TILE, DQ_THREADS>(kc_bh, a.skn, t * BWD_TILE, a.Nk - 1, base, tid);
+    dma_rows<2 * D, BWD_TILE, DQ_THREADS>(v_bh, a.svn * 2, t * BWD_TILE, a.Nk - 1, base + OFF_V, tid);
+    dma_rows<BWD_TILE * 2, D, DQ_THREADS>(blob, BWD_TILE * 2, 0, D - 1, base + OFF_T, tid);
+    dma_flat<WS::CK_BYTES, DQ_THREADS>(blob + WS::T_BYTES, base + OFF_C, tid);
   };
 
   f32x16 dqacc[DB];
@@ -366,69 +322,75 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) dqacc[db][v] = 0.f;
 
-  load_tile(0);
-  for (int t = 0; t < ntiles; ++t) {
-    store_tile();
-    __syncthreads();
-    if (t + 1 < ntiles) load_tile(t + 1);
+  // one 32-key block of tile t
+  auto block = [&](int t, int nb, auto masked_tag) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    const unsigned char *base = smem + (t & 1) * BUF;
+    const unsigned *dgp = reinterpret_cast<const unsigned *>(base + OFF_C);
+    const float *skp = reinterpret_cast<const float *>(base + OFF_C) + 2 * BWD_TILE;
+    const int j0 = t * BWD_TILE;
+    i32x16 acc;
+    f32x16 dp;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { acc[v] = 0; dp[v] = 0.f; }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const i32x4 kf = *reinterpret_cast<const i32x4 *>(base + SK::off(32 * nb + lr, 2 * ks + g));
+      acc = mfma_i8(kf, qf[ks], acc);
+    }
+#pragma unroll
+    for (int kd = 0; kd < KD; ++kd) {
+      const u32x4 vf = *reinterpret_cast<const u32x4 *>(base + OFF_V + SV::off(32 * nb + lr, 2 * kd + g));
+      dp = mfma_16b<T>(vf, dof[kd], dp);
+    }
+    f32x16 f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) f[v] = (float)acc[v];
+    const u32x4 corr_k = {dgp[2 * (32 * nb + lr) + g], 0u, 0u, 0u};
+    f = mfma_16b<T>(corr_k, corr_q, f);
+    float ds[16];
+#pragma unroll
+    for (int aa = 0; aa < 4; ++aa) {
+      const int jl = 32 * nb + 8 * aa + 4 * g;
+      const f32x4 sk4 = *reinterpret_cast<const f32x4 *>(skp + jl);
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) {
+        const int v = 4 * aa + bb;
+        float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, f[v] * sk4[bb], nlse2));
+        if (MASKED) {
+          const int j = j0 + jl + bb;
+          if ((CAUSAL && j > qi) || j >= a.Nk) p = 0.f;
+        }
+        ds[v] = p * (dp[v] - delta_i) * sk4[bb];
+      }
+    }
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      u32x4 dsf;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dsf[e] = pack2<T>(ds[8 * hh + 2 * e], ds[8 * hh + 2 * e + 1]);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const u32x4 ktf = *reinterpret_cast<const u32x4 *>(base + OFF_T + ST::off(32 * db + lr, 4 * nb + 2 * hh + g));
+        dqacc[db] = mfma_16b<T>(ktf, dsf, dqacc[db]);
+      }
+    }
+  };
 
-    const unsigned *dgp = reinterpret_cast<const unsigned *>(smem + OFF_C);
-    const float *skp = reinterpret_cast<const float *>(smem + OFF_C) + 2 * BWD_TILE;
+  load_tile(0);
+  dma_wait();
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    if (t + 1 < ntiles) load_tile(t + 1);
     const int j0 = t * BWD_TILE;
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
       const int jb = j0 + 32 * nb;
-      const bool on = (jb < a.Nk) && (!CAUSAL || jb <= q_last);
-      if (!on) continue;
-      i32x16 acc;
-      f32x16 dp;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) { acc[v] = 0; dp[v] = 0.f; }
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const i32x4 kf = *reinterpret_cast<const i32x4 *>(smem + (32 * nb + lr) * SM::CSTR + ks * 32 + g * 16);
-        acc = mfma_i8(kf, qf[ks], acc);
-      }
-#pragma unroll
-      for (int kd = 0; kd < KD; ++kd) {
-        const u32x4 vf = *reinterpret_cast<const u32x4 *>(smem + OFF_V + (32 * nb + lr) * SM::RSTR + kd * 32 + g * 16);
-        dp = mfma_16b<T>(vf, dof[kd], dp);
-      }
-      f32x16 f;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) f[v] = (float)acc[v];
-      const u32x4 corr_k = {dgp[2 * (32 * nb + lr) + g], 0u, 0u, 0u};
-      f = mfma_16b<T>(corr_k, corr_q, f);
-      const bool need_mask = (CAUSAL && jb + 31 > q_first) || (jb + 32 > a.Nk);
-      float ds[16];
-#pragma unroll
-      for (int aa = 0; aa < 4; ++aa) {
-        const int jl = 32 * nb + 8 * aa + 4 * g;
-        const f32x4 sk4 = *reinterpret_cast<const f32x4 *>(skp + jl);
-#pragma unroll
-        for (int bb = 0; bb < 4; ++bb) {
-          const int v = 4 * aa + bb;
-          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, f[v] * sk4[bb], nlse2));
-          if (need_mask) {
-            const int j = j0 + jl + bb;
-            if ((CAUSAL && j > qi) || j >= a.Nk) p = 0.f;
-          }
-          ds[v] = p * (dp[v] - delta_i) * sk4[bb];
-        }
-      }
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
-        u32x4 dsf;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) dsf[e] = pack2<T>(ds[8 * hh + 2 * e], ds[8 * hh + 2 * e + 1]);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const u32x4 ktf = *reinterpret_cast<const u32x4 *>(smem + OFF_T + (32 * db + lr) * SM::TSTR +
-                                                             (32 * nb + 16 * hh + 8 * g) * 2);
-          dqacc[db] = mfma_16b<T>(ktf, dsf, dqacc[db]);
-        }
-      }
+      if ((jb >= a.Nk) || (CAUSAL && jb > q_last)) continue;               // wave-uniform
+      if ((CAUSAL && jb + 31 > q_first) || (jb + 32 > a.Nk)) block(t, nb, std::true_type{});
+      else block(t, nb, std::false_type{});
     }
+    dma_wait();
     __syncthreads();
   }
 
@@ -449,14 +411,14 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(BwdArgs a) {
 // ------------------------------------------------------------------------------------------ dK, dV
 template <typename T, int D, bool CAUSAL>
 __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
-  typedef BwdSmem<D> SM;
   typedef BwdWs<D> WS;
+  typedef Swz<D> SQ;            // Q code rows
+  typedef Swz<2 * D> SG;        // dO rows
+  typedef Swz<BWD_TILE * 2> ST; // transposed rows
   constexpr int KS = D / 32, DB = D / 32, KD = D / 16;
-  constexpr int QCH = (BWD_TILE * D / 16 + 255) / 256;
-  constexpr int GCH = (BWD_TILE * 2 * D / 16 + 255) / 256;
-  constexpr int TCH = (D * BWD_TILE * 2 / 16 + 255) / 256;
-  constexpr int OFF_DO = SM::C_BYTES, OFF_DOT = OFF_DO + SM::R_BYTES, OFF_QT = OFF_DOT + SM::T_BYTES,
-                OFF_C = OFF_QT + SM::T_BYTES, BUF = OFF_C + WS::CQ_BYTES;
+  constexpr int Q_BYTES = BWD_TILE * D, G_BYTES = BWD_TILE * 2 * D, T_BYTES = WS::T_BYTES;
+  constexpr int OFF_DO = Q_BYTES, OFF_DOT = OFF_DO + G_BYTES, OFF_QT = OFF_DOT + T_BYTES, OFF_C = OFF_QT + T_BYTES,
+                BUF = OFF_C + WS::CQ_BYTES;
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF];
 
   const int L = blockIdx.x;
@@ -497,26 +459,14 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
   const int it0 = CAUSAL ? n0 / BWD_TILE : 0;
   const int ntiles = a.tiles_q;
 
-  Stage<QCH> st_q;
-  Stage<GCH> st_g;
-  Stage<TCH> st_gt, st_qt;
-  u32x4 st_c;
   auto load_tile = [&](int t) {
-    const int i0 = t * BWD_TILE;
+    unsigned char *base = smem + (t & 1) * BUF;
     const unsigned char *blob = wsq_bh + (int64_t)t * WS::Q_BLOB;
-    st_q.load(qc_bh, a.sqn, BWD_TILE, D, i0, a.Nq - 1, tid);
-    st_g.load(do_bh, a.sdon * 2, BWD_TILE, 2 * D, i0, a.Nq - 1, tid);
-    st_gt.load(blob, BWD_TILE * 2, D, BWD_TILE * 2, 0, D - 1, tid);
-    st_qt.load(blob + WS::T_BYTES, BWD_TILE * 2, D, BWD_TILE * 2, 0, D - 1, tid);
-    if (tid < WS::CQ_BYTES / 16) st_c = *reinterpret_cast<const u32x4 *>(blob + 2 * WS::T_BYTES + tid * 16);
-  };
-  auto store_tile = [&](int buf) {
-    unsigned char *base = smem + buf * BUF;
-    st_q.store(base, SM::CSTR, BWD_TILE, D, tid);
-    st_g.store(base + OFF_DO, SM::RSTR, BWD_TILE, 2 * D, tid);
-    st_gt.store(base + OFF_DOT, SM::TSTR, D, BWD_TILE * 2, tid);
-    st_qt.store(base + OFF_QT, SM::TSTR, D, BWD_TILE * 2, tid);
-    if (tid < WS::CQ_BYTES / 16) *reinterpret_cast<u32x4 *>(base + OFF_C + tid * 16) = st_c;
+    dma_rows<D, BWD_TILE, 256>(qc_bh, a.sqn, t * BWD_TILE, a.Nq - 1, base, tid);
+    dma_rows<2 * D, BWD_TILE, 256>(do_bh, a.sdon * 2, t * BWD_TILE, a.Nq - 1, base + OFF_DO, tid);
+    dma_rows<BWD_TILE * 2, D, 256>(blob, BWD_TILE * 2, 0, D - 1, base + OFF_DOT, tid);
+    dma_rows<BWD_TILE * 2, D, 256>(blob + WS::T_BYTES, BWD_TILE * 2, 0, D - 1, base + OFF_QT, tid);
+    dma_flat<WS::CQ_BYTES, 256>(blob + 2 * WS::T_BYTES, base + OFF_C, tid);
   };
 
   f32x16 dkacc[DB], dvacc[DB];
@@ -525,81 +475,84 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) { dkacc[db][v] = 0.f; dvacc[db][v] = 0.f; }
 
-  if (it0 < ntiles) {
-    load_tile(it0);
-    store_tile(it0 & 1);
-  }
-  __syncthreads();
-  for (int t = it0; t < ntiles; ++t) {
-    if (t + 1 < ntiles) load_tile(t + 1);
-
+  // one 32-query block of tile t
+  auto block = [&](int t, int mbk, auto masked_tag) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
     const unsigned char *base = smem + (t & 1) * BUF;
     const unsigned *dgp = reinterpret_cast<const unsigned *>(base + OFF_C);
     const float *cs = reinterpret_cast<const float *>(base + OFF_C);
     const int i0 = t * BWD_TILE;
+    i32x16 acc;
+    f32x16 dp;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { acc[v] = 0; dp[v] = 0.f; }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const i32x4 qfr = *reinterpret_cast<const i32x4 *>(base + SQ::off(32 * mbk + lr, 2 * ks + g));
+      acc = mfma_i8(qfr, kf[ks], acc);
+    }
+#pragma unroll
+    for (int kd = 0; kd < KD; ++kd) {
+      const u32x4 gf = *reinterpret_cast<const u32x4 *>(base + OFF_DO + SG::off(32 * mbk + lr, 2 * kd + g));
+      dp = mfma_16b<T>(gf, vf[kd], dp);
+    }
+    f32x16 f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) f[v] = (float)acc[v];
+    const u32x4 corr_q = {dgp[2 * (32 * mbk + lr) + g], 0u, 0u, 0u};
+    f = mfma_16b<T>(corr_q, corr_k, f);
+    float pp[16], ds[16];
+#pragma unroll
+    for (int aa = 0; aa < 4; ++aa) {
+      const int il = 32 * mbk + 8 * aa + 4 * g;
+      const f32x4 a4 = *reinterpret_cast<const f32x4 *>(cs + 2 * BWD_TILE + il);
+      const f32x4 nl4 = *reinterpret_cast<const f32x4 *>(cs + 3 * BWD_TILE + il);
+      const f32x4 dl4 = *reinterpret_cast<const f32x4 *>(cs + 4 * BWD_TILE + il);
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) {
+        const int v = 4 * aa + bb;
+        float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a4[bb], f[v] * sk_j, nl4[bb]));
+        if (MASKED) {
+          const int i = i0 + il + bb;
+          if ((CAUSAL && kj > i) || i >= a.Nq || kj >= a.Nk) p = 0.f;
+        }
+        pp[v] = p;
+        ds[v] = p * (dp[v] - dl4[bb]) * a4[bb];   // dS * sq * sm_scale * log2(e)
+      }
+    }
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      u32x4 pf, dsf;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        pf[e] = pack2<T>(pp[8 * hh + 2 * e], pp[8 * hh + 2 * e + 1]);
+        dsf[e] = pack2<T>(ds[8 * hh + 2 * e], ds[8 * hh + 2 * e + 1]);
+      }
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int off = ST::off(32 * db + lr, 4 * mbk + 2 * hh + g);
+        const u32x4 gtf = *reinterpret_cast<const u32x4 *>(base + OFF_DOT + off);
+        dvacc[db] = mfma_16b<T>(gtf, pf, dvacc[db]);
+        const u32x4 qtf = *reinterpret_cast<const u32x4 *>(base + OFF_QT + off);
+        dkacc[db] = mfma_16b<T>(qtf, dsf, dkacc[db]);
+      }
+    }
+  };
+
+  if (it0 < ntiles) load_tile(it0);
+  dma_wait();
+  __syncthreads();
+  for (int t = it0; t < ntiles; ++t) {
+    if (t + 1 < ntiles) load_tile(t + 1);
+    const int i0 = t * BWD_TILE;
 #pragma unroll
     for (int mbk = 0; mbk < 2; ++mbk) {
       const int ib = i0 + 32 * mbk;
-      const bool on = (ib < a.Nq) && (!CAUSAL || ib + 31 >= k_first);
-      if (!on) continue;
-      i32x16 acc;
-      f32x16 dp;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) { acc[v] = 0; dp[v] = 0.f; }
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const i32x4 qfr = *reinterpret_cast<const i32x4 *>(base + (32 * mbk + lr) * SM::CSTR + ks * 32 + g * 16);
-        acc = mfma_i8(qfr, kf[ks], acc);
-      }
-#pragma unroll
-      for (int kd = 0; kd < KD; ++kd) {
-        const u32x4 gf = *reinterpret_cast<const u32x4 *>(base + OFF_DO + (32 * mbk + lr) * SM::RSTR + kd * 32 + g * 16);
-        dp = mfma_16b<T>(gf, vf[kd], dp);
-      }
-      f32x16 f;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) f[v] = (float)acc[v];
-      const u32x4 corr_q = {dgp[2 * (32 * mbk + lr) + g], 0u, 0u, 0u};
-      f = mfma_16b<T>(corr_q, corr_k, f);
-      const bool need_mask = (CAUSAL && ib < k_last) || (ib + 32 > a.Nq) || (k_last >= a.Nk);
-      float pp[16], ds[16];
-#pragma unroll
-      for (int aa = 0; aa < 4; ++aa) {
-        const int il = 32 * mbk + 8 * aa + 4 * g;
-        const f32x4 a4 = *reinterpret_cast<const f32x4 *>(cs + 2 * BWD_TILE + il);
-        const f32x4 nl4 = *reinterpret_cast<const f32x4 *>(cs + 3 * BWD_TILE + il);
-        const f32x4 dl4 = *reinterpret_cast<const f32x4 *>(cs + 4 * BWD_TILE + il);
-#pragma unroll
-        for (int bb = 0; bb < 4; ++bb) {
-          const int v = 4 * aa + bb;
-          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a4[bb], f[v] * sk_j, nl4[bb]));
-          if (need_mask) {
-            const int i = i0 + il + bb;
-            if ((CAUSAL && kj > i) || i >= a.Nq || kj >= a.Nk) p = 0.f;
-          }
-          pp[v] = p;
-          ds[v] = p * (dp[v] - dl4[bb]) * a4[bb];   // dS * sq * sm_scale * log2(e)
-        }
-      }
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
-        u32x4 pf, dsf;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          pf[e] = pack2<T>(pp[8 * hh + 2 * e], pp[8 * hh + 2 * e + 1]);
-          dsf[e] = pack2<T>(ds[8 * hh + 2 * e], ds[8 * hh + 2 * e + 1]);
-        }
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const int off = (32 * db + lr) * SM::TSTR + (32 * mbk + 16 * hh + 8 * g) * 2;
-          const u32x4 gtf = *reinterpret_cast<const u32x4 *>(base + OFF_DOT + off);
-          dvacc[db] = mfma_16b<T>(gtf, pf, dvacc[db]);
-          const u32x4 qtf = *reinterpret_cast<const u32x4 *>(base + OFF_QT + off);
-          dkacc[db] = mfma_16b<T>(qtf, dsf, dkacc[db]);
-        }
-      }
+      if ((ib >= a.Nq) || (CAUSAL && ib + 31 < k_first)) continue;          // wave-uniform
+      if ((CAUSAL && ib < k_last) || (ib + 32 > a.Nq) || (k_last >= a.Nk)) block(t, mbk, std::true_type{});
+      else block(t, mbk, std::false_type{});
     }
-    if (t + 1 < ntiles) store_tile((t + 1) & 1);
+    dma_wait();
     __syncthreads();
   }
 
@@ -660,14 +613,14 @@ template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStre
   }
   // dQ
   {
-    a.nblocks = (int)((x.Nq + BWD_BLK - 1) / BWD_BLK);
+    a.nblocks = (int)((x.Nq + DQ_BLK - 1) / DQ_BLK);
     const int64_t total = (int64_t)a.nblocks * BH;
     if (total > 0x3fffffffLL) return set_error(QFA_EUNSUPPORTED, "attn_bwd: too many query blocks for one launch");
     a.total_blocks = (int)total;
     a.blocks_per_xcd = (a.total_blocks + 7) / 8;
     const dim3 grid((unsigned)(a.blocks_per_xcd * 8));
-    if (x.causal) bwd_dq_kernel<T, D, true><<<grid, block, 0, st>>>(a);
-    else bwd_dq_kernel<T, D, false><<<grid, block, 0, st>>>(a);
+    if (x.causal) bwd_dq_kernel<T, D, true><<<grid, dim3(DQ_THREADS), 0, st>>>(a);
+    else bwd_dq_kernel<T, D, false><<<grid, dim3(DQ_THREADS), 0, st>>>(a);
     if (int e = check_launch("qfa_attn_bwd (dq)")) return e;
   }
   return 0;

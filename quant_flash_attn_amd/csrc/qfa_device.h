@@ -92,4 +92,53 @@ template <int CTRL> __device__ __forceinline__ int dpp_i(int x) {
 // value held by lane (l ^ 32)
 __device__ __forceinline__ float swap32_f(float x) { return __shfl_xor(x, 32, 64); }
 
+// ---- direct global -> LDS tile copies -------------------------------------------------------------
+// global_load_lds_dwordx4 writes lane l's 16 bytes to LDS[wave-uniform base + 16*l], so a tile lands
+// in LDS as dense rows without padding.  Bank conflicts are avoided by an XOR swizzle applied on the
+// global side: the 16-byte slot (row r, position q) holds the row's chunk q ^ swz(r), with swz
+// chosen so that 16 consecutive rows read at the same logical chunk hit 16 different 16-byte slots
+// of the 256-byte bank line.
+template <int ROW_BYTES> struct Swz {
+  static constexpr int CPR = ROW_BYTES / 16;                 // chunks per row (4, 8 or 16)
+  static constexpr int RP = 16 / CPR;                        // rows per 256 bytes
+  static __device__ __forceinline__ int swz(int row) { return (row / RP) % CPR; }
+  // byte offset of logical chunk c of row r inside the tile
+  static __device__ __forceinline__ int off(int r, int c) { return r * ROW_BYTES + ((c ^ swz(r)) << 4); }
+};
+
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+// rows [row0, row0+ROWS) (clamped to row_max) of a row-major global array -> swizzled LDS tile; NT threads
+template <int ROW_BYTES, int ROWS, int NT>
+__device__ __forceinline__ void dma_rows(const unsigned char *g, int64_t gstride, int row0, int row_max,
+                                         unsigned char *lds, int tid) {
+  typedef Swz<ROW_BYTES> S;
+  constexpr int TOTAL = ROWS * S::CPR;
+#pragma unroll
+  for (int i = 0; i < (TOTAL + NT - 1) / NT; ++i) {
+    const int p = tid + NT * i;
+    if (TOTAL % NT == 0 || p < TOTAL) {
+      const int row = p / S::CPR, pos = p % S::CPR;
+      const int c = pos ^ S::swz(row);
+      const int rr = min(row0 + row, row_max);
+      __builtin_amdgcn_global_load_lds((gptr_t)(g + (int64_t)rr * gstride + c * 16),
+                                       (lptr_t)(lds + ((tid & ~63) + NT * i) * 16), 16, 0, 0);
+    }
+  }
+}
+// BYTES contiguous bytes, copied as they are
+template <int BYTES, int NT>
+__device__ __forceinline__ void dma_flat(const unsigned char *g, unsigned char *lds, int tid) {
+  constexpr int TOTAL = BYTES / 16;
+#pragma unroll
+  for (int i = 0; i < (TOTAL + NT - 1) / NT; ++i) {
+    const int p = tid + NT * i;
+    if (TOTAL % NT == 0 || p < TOTAL)
+      __builtin_amdgcn_global_load_lds((gptr_t)(g + p * 16), (lptr_t)(lds + ((tid & ~63) + NT * i) * 16), 16, 0, 0);
+  }
+}
+// all direct loads of this wave have landed (vmcnt(0)); follow with a barrier before other waves read
+__device__ __forceinline__ void dma_wait() { __builtin_amdgcn_s_waitcnt(0x0f70); }
+
 }  // namespace qfa
