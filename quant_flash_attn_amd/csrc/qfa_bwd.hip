@@ -409,8 +409,20 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(BwdArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------ dK, dV
+// One workgroup = 128 keys = 8 waves.  The dK^T and dV^T accumulators of 32 keys take 128 registers,
+// too many for two waves per SIMD, so each 32-key slice is shared by a PAIR of waves that sit on the
+// same SIMD (waves w and w+4):
+//   P-wave  (w < 4):  S = Qc.Kc^T (INT8 MFMA), P = exp2(.), hands P to its partner through LDS,
+//                     dV^T += dO^T.P
+//   dS-wave (w >= 4): dP = dO.V^T, then dS' = P o (dP - delta) * a with the partner's P,
+//                     dK^T += Qz^T.dS'
+// No product is computed twice, each wave keeps 64 accumulator registers, and within a SIMD one wave
+// is in its VALU phase while the other feeds the matrix pipe.  Two barriers per 32-query block: after
+// P is written, and after it has been consumed.
+constexpr int DKV_THREADS = 512;
+
 template <typename T, int D, bool CAUSAL>
-__global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
+__global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
   typedef BwdWs<D> WS;
   typedef Swz<D> SQ;            // Q code rows
   typedef Swz<2 * D> SG;        // dO rows
@@ -419,7 +431,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
   constexpr int Q_BYTES = BWD_TILE * D, G_BYTES = BWD_TILE * 2 * D, T_BYTES = WS::T_BYTES;
   constexpr int OFF_DO = Q_BYTES, OFF_DOT = OFF_DO + G_BYTES, OFF_QT = OFF_DOT + T_BYTES, OFF_C = OFF_QT + T_BYTES,
                 BUF = OFF_C + WS::CQ_BYTES;
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF];
+  constexpr int OFF_X = 2 * BUF;             // P exchange: 4 pairs x 64 lanes x 16 floats
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF + 4 * 4096];
 
   const int L = blockIdx.x;
   const int vid = (L % 8) * a.blocks_per_xcd + (L / 8);
@@ -429,6 +442,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
   const int64_t b = bh / a.H, h = bh % a.H;
   const int n0 = nbk * BWD_BLK;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, lr = lane % 32, g = lane / 32;
+  const int pair = wave % 4;
+  const bool p_role = wave < 4;      // wave-uniform
 
   const unsigned char *qc_bh = reinterpret_cast<const unsigned char *>(a.qc + b * a.sqb + h * a.sqh);
   const int8_t *kc_bh = a.kc + b * a.skb + h * a.skh;
@@ -439,22 +454,24 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
   const unsigned char *wsk_bh = a.ws_k + (int64_t)bh * a.tiles_k * WS::K_BLOB;
   const unsigned char *wsq_bh = a.ws_q + (int64_t)bh * a.tiles_q * WS::Q_BLOB;
 
-  // ---- this lane's key
-  const int kj = n0 + wave * 32 + lr;
+  // ---- this lane's key: INT8 codes + correction digits + scale for the P role, V row for the dS role
+  const int kj = n0 + pair * 32 + lr;
   const int kj_c = kj < a.Nk ? kj : a.Nk - 1;
-  i32x4 kf[KS];
+  u32x4 breg[KD];   // persistent B operand: K codes (first KS entries) or V (KD entries)
+  if (p_role) {
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks)
-    kf[ks] = *reinterpret_cast<const i32x4 *>(kc_bh + (int64_t)kj_c * a.skn + ks * 32 + g * 16);
-  u32x4 vf[KD];
+    for (int ks = 0; ks < KS; ++ks)
+      breg[ks] = *reinterpret_cast<const u32x4 *>(kc_bh + (int64_t)kj_c * a.skn + ks * 32 + g * 16);
+  } else {
 #pragma unroll
-  for (int kd = 0; kd < KD; ++kd)
-    vf[kd] = *reinterpret_cast<const u32x4 *>(v_bh + (int64_t)kj_c * a.svn + kd * 16 + g * 8);
+    for (int kd = 0; kd < KD; ++kd)
+      breg[kd] = *reinterpret_cast<const u32x4 *>(v_bh + (int64_t)kj_c * a.svn + kd * 16 + g * 8);
+  }
   const unsigned *ck = reinterpret_cast<const unsigned *>(wsk_bh + (int64_t)(kj_c / BWD_TILE) * WS::K_BLOB + WS::T_BYTES);
   const int kl = kj_c % BWD_TILE;
   const u32x4 corr_k = {ck[2 * kl + g], 0u, 0u, 0u};
   const float sk_j = __builtin_bit_cast(float, ck[2 * BWD_TILE + kl]);
-  const int k_first = n0 + wave * 32, k_last = k_first + 31;
+  const int k_first = n0 + pair * 32, k_last = k_first + 31;
 
   const int it0 = CAUSAL ? n0 / BWD_TILE : 0;
   const int ntiles = a.tiles_q;
@@ -462,114 +479,214 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdArgs a) {
   auto load_tile = [&](int t) {
     unsigned char *base = smem + (t & 1) * BUF;
     const unsigned char *blob = wsq_bh + (int64_t)t * WS::Q_BLOB;
-    dma_rows<D, BWD_TILE, 256>(qc_bh, a.sqn, t * BWD_TILE, a.Nq - 1, base, tid);
-    dma_rows<2 * D, BWD_TILE, 256>(do_bh, a.sdon * 2, t * BWD_TILE, a.Nq - 1, base + OFF_DO, tid);
-    dma_rows<BWD_TILE * 2, D, 256>(blob, BWD_TILE * 2, 0, D - 1, base + OFF_DOT, tid);
-    dma_rows<BWD_TILE * 2, D, 256>(blob + WS::T_BYTES, BWD_TILE * 2, 0, D - 1, base + OFF_QT, tid);
-    dma_flat<WS::CQ_BYTES, 256>(blob + 2 * WS::T_BYTES, base + OFF_C, tid);
+    dma_rows<D, BWD_TILE, DKV_THREADS>(qc_bh, a.sqn, t * BWD_TILE, a.Nq - 1, base, tid);
+    dma_rows<2 * D, BWD_TILE, DKV_THREADS>(do_bh, a.sdon * 2, t * BWD_TILE, a.Nq - 1, base + OFF_DO, tid);
+    dma_rows<BWD_TILE * 2, D, DKV_THREADS>(blob, BWD_TILE * 2, 0, D - 1, base + OFF_DOT, tid);
+    dma_rows<BWD_TILE * 2, D, DKV_THREADS>(blob + WS::T_BYTES, BWD_TILE * 2, 0, D - 1, base + OFF_QT, tid);
+    dma_flat<WS::CQ_BYTES, DKV_THREADS>(blob + 2 * WS::T_BYTES, base + OFF_C, tid);
   };
 
-  f32x16 dkacc[DB], dvacc[DB];
+  f32x16 oacc[DB];   // dV^T (P role) or dK^T (dS role) for this lane's key
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) { dkacc[db][v] = 0.f; dvacc[db][v] = 0.f; }
+    for (int v = 0; v < 16; ++v) oacc[db][v] = 0.f;
 
-  // one 32-query block of tile t
-  auto block = [&](int t, int mbk, auto masked_tag) {
+  f32x4 *xch = reinterpret_cast<f32x4 *>(smem + OFF_X + pair * 4096);   // [4][64 lanes] of 4 floats
+
+  // LDS operands are fetched in groups well ahead of the MFMAs that consume them (a 16-byte LDS read
+  // takes far longer than an MFMA issue slot, and the compiler keeps loads next to their use), the
+  // groups are pinned in place with scheduling barriers.
+  // ---- P role, first half of a block: S, correction, P; P goes to LDS (fp32) and stays packed in pf;
+  // the dO^T fragments of the second half are fetched here as well
+  auto p_first = [&](const unsigned char *base, int i0, int mbk, u32x4 (&pf)[2], u32x4 (&tf)[2 * DB], auto masked_tag) {
     constexpr bool MASKED = decltype(masked_tag)::value;
-    const unsigned char *base = smem + (t & 1) * BUF;
     const unsigned *dgp = reinterpret_cast<const unsigned *>(base + OFF_C);
     const float *cs = reinterpret_cast<const float *>(base + OFF_C);
-    const int i0 = t * BWD_TILE;
-    i32x16 acc;
-    f32x16 dp;
+    i32x4 qfr[KS];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) { acc[v] = 0; dp[v] = 0.f; }
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const i32x4 qfr = *reinterpret_cast<const i32x4 *>(base + SQ::off(32 * mbk + lr, 2 * ks + g));
-      acc = mfma_i8(qfr, kf[ks], acc);
-    }
-#pragma unroll
-    for (int kd = 0; kd < KD; ++kd) {
-      const u32x4 gf = *reinterpret_cast<const u32x4 *>(base + OFF_DO + SG::off(32 * mbk + lr, 2 * kd + g));
-      dp = mfma_16b<T>(gf, vf[kd], dp);
-    }
-    f32x16 f;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) f[v] = (float)acc[v];
+    for (int ks = 0; ks < KS; ++ks)
+      qfr[ks] = *reinterpret_cast<const i32x4 *>(base + SQ::off(32 * mbk + lr, 2 * ks + g));
     const u32x4 corr_q = {dgp[2 * (32 * mbk + lr) + g], 0u, 0u, 0u};
-    f = mfma_16b<T>(corr_q, corr_k, f);
-    float pp[16], ds[16];
+    f32x4 a4[4], nl4[4];
 #pragma unroll
     for (int aa = 0; aa < 4; ++aa) {
       const int il = 32 * mbk + 8 * aa + 4 * g;
-      const f32x4 a4 = *reinterpret_cast<const f32x4 *>(cs + 2 * BWD_TILE + il);
-      const f32x4 nl4 = *reinterpret_cast<const f32x4 *>(cs + 3 * BWD_TILE + il);
-      const f32x4 dl4 = *reinterpret_cast<const f32x4 *>(cs + 4 * BWD_TILE + il);
+      a4[aa] = *reinterpret_cast<const f32x4 *>(cs + 2 * BWD_TILE + il);
+      nl4[aa] = *reinterpret_cast<const f32x4 *>(cs + 3 * BWD_TILE + il);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    i32x16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) acc = mfma_i8(qfr[ks], __builtin_bit_cast(i32x4, breg[ks]), acc);
+    f32x16 f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) f[v] = (float)acc[v];
+    f = mfma_16b<T>(corr_q, corr_k, f);
+    float pp[16];
+#pragma unroll
+    for (int aa = 0; aa < 4; ++aa) {
+      const int il = 32 * mbk + 8 * aa + 4 * g;
+      f32x4 p4;
 #pragma unroll
       for (int bb = 0; bb < 4; ++bb) {
-        const int v = 4 * aa + bb;
-        float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a4[bb], f[v] * sk_j, nl4[bb]));
+        float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a4[aa][bb], f[4 * aa + bb] * sk_j, nl4[aa][bb]));
         if (MASKED) {
           const int i = i0 + il + bb;
           if ((CAUSAL && kj > i) || i >= a.Nq || kj >= a.Nk) p = 0.f;
         }
-        pp[v] = p;
-        ds[v] = p * (dp[v] - dl4[bb]) * a4[bb];   // dS * sq * sm_scale * log2(e)
+        pp[4 * aa + bb] = p;
+        p4[bb] = p;
       }
+      xch[aa * 64 + lane] = p4;
     }
 #pragma unroll
-    for (int hh = 0; hh < 2; ++hh) {
-      u32x4 pf, dsf;
+    for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        pf[e] = pack2<T>(pp[8 * hh + 2 * e], pp[8 * hh + 2 * e + 1]);
-        dsf[e] = pack2<T>(ds[8 * hh + 2 * e], ds[8 * hh + 2 * e + 1]);
-      }
+      for (int e = 0; e < 4; ++e) pf[hh][e] = pack2<T>(pp[8 * hh + 2 * e], pp[8 * hh + 2 * e + 1]);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const int off = ST::off(32 * db + lr, 4 * mbk + 2 * hh + g);
-        const u32x4 gtf = *reinterpret_cast<const u32x4 *>(base + OFF_DOT + off);
-        dvacc[db] = mfma_16b<T>(gtf, pf, dvacc[db]);
-        const u32x4 qtf = *reinterpret_cast<const u32x4 *>(base + OFF_QT + off);
-        dkacc[db] = mfma_16b<T>(qtf, dsf, dkacc[db]);
-      }
+    for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+        tf[hh * DB + db] = *reinterpret_cast<const u32x4 *>(base + OFF_DOT + ST::off(32 * db + lr, 4 * mbk + 2 * hh + g));
+  };
+  // ---- dS role, first half: dP = dO.V^T; then the Qz^T fragments and constants of the second half
+  auto ds_first = [&](const unsigned char *base, int mbk, f32x16 &dp, u32x4 (&tf)[2 * DB], f32x4 (&a4)[4], f32x4 (&dl4)[4]) {
+    const float *cs = reinterpret_cast<const float *>(base + OFF_C);
+    u32x4 gf[KD];
+#pragma unroll
+    for (int kd = 0; kd < KD; ++kd)
+      gf[kd] = *reinterpret_cast<const u32x4 *>(base + OFF_DO + SG::off(32 * mbk + lr, 2 * kd + g));
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dp[v] = 0.f;
+#pragma unroll
+    for (int kd = 0; kd < KD; ++kd) dp = mfma_16b<T>(gf[kd], breg[kd], dp);
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+        tf[hh * DB + db] = *reinterpret_cast<const u32x4 *>(base + OFF_QT + ST::off(32 * db + lr, 4 * mbk + 2 * hh + g));
+#pragma unroll
+    for (int aa = 0; aa < 4; ++aa) {
+      const int il = 32 * mbk + 8 * aa + 4 * g;
+      a4[aa] = *reinterpret_cast<const f32x4 *>(cs + 2 * BWD_TILE + il);
+      dl4[aa] = *reinterpret_cast<const f32x4 *>(cs + 4 * BWD_TILE + il);
     }
   };
+  // ---- second half: accumulate with the prefetched transposed fragments
+  auto accumulate = [&](const u32x4 (&tf)[2 * DB], const u32x4 (&bf)[2]) {
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) oacc[db] = mfma_16b<T>(tf[hh * DB + db], bf[hh], oacc[db]);
+  };
+  // ---- dS role, second half prologue: dS' = P (from partner) * (dP - delta) * a, packed
+  auto ds_second = [&](const f32x16 &dp, const f32x4 (&a4)[4], const f32x4 (&dl4)[4], u32x4 (&dsf)[2]) {
+    f32x4 p4[4];
+#pragma unroll
+    for (int aa = 0; aa < 4; ++aa) p4[aa] = xch[aa * 64 + lane];
+    float ds[16];
+#pragma unroll
+    for (int aa = 0; aa < 4; ++aa)
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) ds[4 * aa + bb] = p4[aa][bb] * (dp[4 * aa + bb] - dl4[aa][bb]) * a4[aa][bb];
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dsf[hh][e] = pack2<T>(ds[8 * hh + 2 * e], ds[8 * hh + 2 * e + 1]);
+  };
 
+#ifdef QFA_TIMING
+  long long tacc[5] = {0, 0, 0, 0, 0};
+  long long tprev = clock64();
+#define QFA_TICK(i) { const long long tn = clock64(); tacc[i] += tn - tprev; tprev = tn; }
+#else
+#define QFA_TICK(i)
+#endif
   if (it0 < ntiles) load_tile(it0);
   dma_wait();
   __syncthreads();
-  for (int t = it0; t < ntiles; ++t) {
-    if (t + 1 < ntiles) load_tile(t + 1);
-    const int i0 = t * BWD_TILE;
+  QFA_TICK(0)
+  // The two roles run separate loops with the same barrier sequence (2 per 32-query block).
+  auto block_flags = [&](int t, int mbk, bool &on, bool &masked) {
+    const int ib = t * BWD_TILE + 32 * mbk;
+    on = (ib < a.Nq) && (!CAUSAL || ib + 31 >= k_first);                               // wave-uniform
+    masked = (CAUSAL && ib < k_last) || (ib + 32 > a.Nq) || (k_last >= a.Nk);
+  };
+  if (p_role) {
+    for (int t = it0; t < ntiles; ++t) {
+      if (t + 1 < ntiles) load_tile(t + 1);
+      const unsigned char *base = smem + (t & 1) * BUF;
 #pragma unroll
-    for (int mbk = 0; mbk < 2; ++mbk) {
-      const int ib = i0 + 32 * mbk;
-      if ((ib >= a.Nq) || (CAUSAL && ib + 31 < k_first)) continue;          // wave-uniform
-      if ((CAUSAL && ib < k_last) || (ib + 32 > a.Nq) || (k_last >= a.Nk)) block(t, mbk, std::true_type{});
-      else block(t, mbk, std::false_type{});
+      for (int mbk = 0; mbk < 2; ++mbk) {
+        bool on, masked;
+        block_flags(t, mbk, on, masked);
+        u32x4 pf[2], tf[2 * DB];
+        QFA_TICK(0)
+        if (on) {
+          if (masked) p_first(base, t * BWD_TILE, mbk, pf, tf, std::true_type{});
+          else p_first(base, t * BWD_TILE, mbk, pf, tf, std::false_type{});
+        }
+        QFA_TICK(1)
+        lds_barrier();   // P of this block is in LDS (the next tile's direct loads stay in flight)
+        QFA_TICK(2)
+        if (on) accumulate(tf, pf);
+        QFA_TICK(3)
+        if (mbk == 1) dma_wait();
+        lds_barrier();   // P consumed; after the second block the next tile has landed
+        QFA_TICK(4)
+      }
     }
-    dma_wait();
-    __syncthreads();
+  } else {
+    for (int t = it0; t < ntiles; ++t) {
+      if (t + 1 < ntiles) load_tile(t + 1);
+      const unsigned char *base = smem + (t & 1) * BUF;
+#pragma unroll
+      for (int mbk = 0; mbk < 2; ++mbk) {
+        bool on, masked;
+        block_flags(t, mbk, on, masked);
+        u32x4 dsf[2], tf[2 * DB];
+        f32x16 dp;
+        f32x4 a4[4], dl4[4];
+        QFA_TICK(0)
+        if (on) ds_first(base, mbk, dp, tf, a4, dl4);
+        QFA_TICK(1)
+        lds_barrier();
+        QFA_TICK(2)
+        if (on) {
+          ds_second(dp, a4, dl4, dsf);
+          accumulate(tf, dsf);
+        }
+        QFA_TICK(3)
+        if (mbk == 1) dma_wait();
+        lds_barrier();
+        QFA_TICK(4)
+      }
+    }
   }
+#ifdef QFA_TIMING
+  if (lane == 0 && bh == 0) {
+    long long *out = reinterpret_cast<long long *>(a.dq) + (nbk * 8 + wave) * 8;
+    for (int i = 0; i < 5; ++i) out[i] = tacc[i];
+    out[5] = ntiles - it0;
+  }
+#endif
 
   if (kj < a.Nk) {
-    T *krow = dk_bh + (int64_t)kj * a.sdkn;
-    T *vrow = dv_bh + (int64_t)kj * a.sdvn;
+    T *row = (p_role ? dv_bh + (int64_t)kj * a.sdvn : dk_bh + (int64_t)kj * a.sdkn);
+    const float scale = p_role ? 1.0f : kLn2;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa) {
         u32x2 w;
-        w[0] = pack2<T>(dkacc[db][4 * aa + 0] * kLn2, dkacc[db][4 * aa + 1] * kLn2);
-        w[1] = pack2<T>(dkacc[db][4 * aa + 2] * kLn2, dkacc[db][4 * aa + 3] * kLn2);
-        *reinterpret_cast<u32x2 *>(krow + 32 * db + 8 * aa + 4 * g) = w;
-        w[0] = pack2<T>(dvacc[db][4 * aa + 0], dvacc[db][4 * aa + 1]);
-        w[1] = pack2<T>(dvacc[db][4 * aa + 2], dvacc[db][4 * aa + 3]);
-        *reinterpret_cast<u32x2 *>(vrow + 32 * db + 8 * aa + 4 * g) = w;
+        w[0] = pack2<T>(oacc[db][4 * aa + 0] * scale, oacc[db][4 * aa + 1] * scale);
+        w[1] = pack2<T>(oacc[db][4 * aa + 2] * scale, oacc[db][4 * aa + 3] * scale);
+        *reinterpret_cast<u32x2 *>(row + 32 * db + 8 * aa + 4 * g) = w;
       }
   }
 }
@@ -607,8 +724,8 @@ template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStre
     a.total_blocks = (int)total;
     a.blocks_per_xcd = (a.total_blocks + 7) / 8;
     const dim3 grid((unsigned)(a.blocks_per_xcd * 8));
-    if (x.causal) bwd_dkdv_kernel<T, D, true><<<grid, block, 0, st>>>(a);
-    else bwd_dkdv_kernel<T, D, false><<<grid, block, 0, st>>>(a);
+    if (x.causal) bwd_dkdv_kernel<T, D, true><<<grid, dim3(DKV_THREADS), 0, st>>>(a);
+    else bwd_dkdv_kernel<T, D, false><<<grid, dim3(DKV_THREADS), 0, st>>>(a);
     if (int e = check_launch("qfa_attn_bwd (dk, dv)")) return e;
   }
   // dQ
@@ -619,8 +736,10 @@ template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStre
     a.total_blocks = (int)total;
     a.blocks_per_xcd = (a.total_blocks + 7) / 8;
     const dim3 grid((unsigned)(a.blocks_per_xcd * 8));
+#ifndef QFA_TIMING
     if (x.causal) bwd_dq_kernel<T, D, true><<<grid, dim3(DQ_THREADS), 0, st>>>(a);
     else bwd_dq_kernel<T, D, false><<<grid, dim3(DQ_THREADS), 0, st>>>(a);
+#endif
     if (int e = check_launch("qfa_attn_bwd (dq)")) return e;
   }
   return 0;

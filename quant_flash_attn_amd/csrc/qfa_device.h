@@ -140,5 +140,9 @@ __device__ __forceinline__ void dma_flat(const unsigned char *g, unsigned char *
 }
 // all direct loads of this wave have landed (vmcnt(0)); follow with a barrier before other waves read
 __device__ __forceinline__ void dma_wait() { __builtin_amdgcn_s_waitcnt(0x0f70); }
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
+// global access, including direct-to-LDS loads issued for a LATER tile, which would serialise the
+// prefetch; this one leaves them in flight (pair it with dma_wait() where a tile must have landed).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 }  // namespace qfa
