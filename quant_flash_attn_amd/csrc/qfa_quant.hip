@@ -11,8 +11,9 @@
 // load per lane for 16-bit inputs, two for fp32), so one wave64 load instruction covers
 // 512/D tokens with fully coalesced 16-byte accesses.  The row is read once, kept in
 // registers, reduced with DPP lane permutes inside the lane group (no LDS), and the codes
-// leave as one 8-byte store per lane.  HBM-bound: D*sizeof(in) + D + 9 bytes per token
-// (+2 with the 16-bit scale copy).
+// leave as one 8-byte store per lane.  HBM-bound in principle (D*sizeof(in) + D + 9 bytes per token,
+// +2 with the 16-bit scale copy); in practice the exact arithmetic makes VALU issue the limiter, so
+// the per-element instruction count is kept low (see the division and packing notes below).
 #include "qfa_device.h"
 #include "qfa_host.h"
 
@@ -116,21 +117,54 @@ template <typename T, int D, int U> __global__ __launch_bounds__(256) void quant
     mx = group_max<LPT>(mx);
     float scale = (mx - mn) / 255.0f;
     scale = (scale == 0.0f) ? 1.0f : scale;
-    const float zpf = -128.0f - mn / scale;
-    const float zp = fmaxf(-128.0f, fminf(127.0f, __builtin_roundf(zpf)));
-    int c[8];
-    int sum = 0;
+    // Division by the per-token scale.  In the common exponent range the quotient is formed with the
+    // same FMA refinement the hardware division sequence uses (reciprocal refined once, two residual
+    // corrections of the quotient), which gives the correctly rounded x/scale without the per-element
+    // operand scaling; outside that range (tiny scale, huge values, NaN) the IEEE `/` is used.
+    // Quotients below 2^-30 in magnitude may differ in their last bits, which cannot matter: they
+    // vanish in the addition of the zero point or round to zero.
+    const bool fast = (scale >= 0x1p-60f) && (fmaxf(fabsf(mn), fabsf(mx)) <= 0x1p60f);
+    float r = __builtin_amdgcn_rcpf(scale);
+    r = __builtin_fmaf(__builtin_fmaf(-scale, r, 1.0f), r, r);
+    auto fdiv = [&](float x) -> float {
+      float q = x * r;
+      q = __builtin_fmaf(__builtin_fmaf(-scale, q, x), r, q);
+      q = __builtin_fmaf(__builtin_fmaf(-scale, q, x), r, q);
+      return q;
+    };
+    // roundf (ties away from zero): trunc, exact fraction, compare with one half
+    auto round_away = [](float y) -> float {
+      const float t = __builtin_truncf(y);
+      const float d = y - t;
+      return (fabsf(d) >= 0.5f) ? t + __builtin_copysignf(1.0f, y) : t;
+    };
+    float q[8], qmn;
+    if (fast) {
+      qmn = fdiv(mn);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) q[e] = fdiv(v[u][e]);
+    } else {
+      qmn = mn / scale;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) q[e] = v[u][e] / scale;
+    }
+    const float zpf = -128.0f - qmn;
+    const float zp = fmaxf(-128.0f, fminf(127.0f, round_away(zpf)));
+    // codes leave as biased bytes: roundf(.) + 128 converted with unsigned saturation (= the clamp to
+    // [-128, 127]), flipped back to two's complement with one XOR per dword
+    u32x2 w = {0u, 0u};
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const float y = v[u][e] / scale + zp;
-      c[e] = (int)fmaxf(-128.0f, fminf(127.0f, __builtin_roundf(y)));
-      sum += c[e];
+      const float y = q[e] + zp;
+      const float c = round_away(y) + 128.0f;
+      w[e / 4] = __builtin_amdgcn_cvt_pk_u8_f32(c, e % 4, w[e / 4]);
     }
+    int sum = (int)__builtin_amdgcn_sad_u8(w[0], 0u, 0u);
+    sum = (int)__builtin_amdgcn_sad_u8(w[1], 0u, (unsigned)sum) - 8 * 128;
+    w[0] ^= 0x80808080u;
+    w[1] ^= 0x80808080u;
     sum = group_sum<LPT>(sum);
     if (live[u]) {
-      u32x2 w;
-      w[0] = (c[0] & 0xff) | ((c[1] & 0xff) << 8) | ((c[2] & 0xff) << 16) | ((unsigned)c[3] << 24);
-      w[1] = (c[4] & 0xff) | ((c[5] & 0xff) << 8) | ((c[6] & 0xff) << 16) | ((unsigned)c[7] << 24);
       *reinterpret_cast<u32x2 *>(cb + n * a.scn + sub * 8) = w;
       if (sub == 0) {
         const int64_t t = bh * a.N + n;

@@ -52,6 +52,21 @@ def test_ties_saturation_and_constant_rows(qfa):
     assert got.zero_point[0, 0, 1].item() == -117
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_wide_exponent_range(qfa, dtype):
+    """Tokens scaled by 2^k, k in [-75, 75]: exercises both division paths of the kernel (the FMA
+    refinement used in the common exponent range and the IEEE division outside it), plus rows whose
+    range is far smaller than their offset."""
+    g = torch.Generator().manual_seed(11)
+    B, H, N, D = 2, 4, 4096, 128
+    x = torch.randn(B, H, N, D, generator=g)
+    k = torch.randint(-75, 76, (B, H, N, 1), generator=g).float()
+    x = x * torch.exp2(k)
+    x[0, 0, ::7] = 1.0 + x[0, 0, ::7].sign() * 1e-5          # tiny range on a large offset
+    x[0, 1, ::5] += 300.0                                     # all-positive rows, zero point clamps
+    _check(qfa, x.to(dtype), "wide exponent range")
+
+
 def test_strided_input(qfa):
     """[B,N,H,D] storage viewed as [B,H,N,D] (the usual projection layout)."""
     base = torch.randn(2, 300, 4, 128, generator=torch.Generator().manual_seed(9)).to(torch.bfloat16)
