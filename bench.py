@@ -166,9 +166,14 @@ def main():
     extra["fwd_bwd_ms_incl_quant"] = round(ms_step + ms_bwd, 4)
     extra["fwd_bwd_tflops_incl_quant"] = round((F_fwd + F_bwd) / ((ms_step + ms_bwd) * 1e-3) / 1e12, 2)
     extra["fwd_bwd_tflops_kernels_only"] = round((F_fwd + F_bwd) / ((ms_fwd_only + ms_bwd) * 1e-3) / 1e12, 2)
-    # the QK^T product is half of the forward FLOPs and runs on INT8 MFMA
+    # the QK^T product is half of the forward FLOPs and runs on INT8 MFMA: over the whole kernel, and over
+    # the QK^T stage alone (same kernel with the exponentials and P.V compiled out)
     extra["qk_int8_tops_over_whole_fwd_kernel"] = round(0.5 * F_fwd / (ms_fwd_only * 1e-3) / 1e12, 2)
     extra["qk_frac_int8_peak_over_whole_fwd_kernel"] = round(0.5 * F_fwd / (ms_fwd_only * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)
+    ms_qk = time_events(lambda: qfa.attn_fwd_quantized(qq, kq, v, causal, sm, _entry="qfa_bench_qk_stage"), args.steps, 5)
+    extra["qk_stage_ms"] = round(ms_qk, 4)
+    extra["qk_stage_int8_tops"] = round(0.5 * F_fwd / (ms_qk * 1e-3) / 1e12, 2)
+    extra["qk_stage_frac_int8_peak"] = round(0.5 * F_fwd / (ms_qk * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)
 
     if args.sdpa:
         import torch.nn.functional as Fn

@@ -92,6 +92,19 @@ int qfa_attn_fwd(const int8_t *qc, const float *sq, const int8_t *zq, const int3
                  int64_t sob, int64_t soh, int64_t son, float sm_scale, int causal, void *stream);
 
 /*
+ * Measurement hook, same arguments as qfa_attn_fwd: runs the forward kernel with the exponentials
+ * and the P.V product compiled out (same K/V/Q loads, INT8 QK^T MFMAs, zero-point correction, key
+ * scaling and running row maximum).  O is left untouched; lse receives the scaled row maxima.
+ * Used by bench.py to time the QK^T stage alone against the INT8 MFMA peak; no counterpart in
+ * the reference (its compute_flops.py:89-151 times whole kernels only).
+ */
+int qfa_bench_qk_stage(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,
+                       const float *sk, const int8_t *zk, const int32_t *rk, const void *v, void *o, float *lse,
+                       int io_dtype, int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D, int64_t sqb, int64_t sqh,
+                       int64_t sqn, int64_t skb, int64_t skh, int64_t skn, int64_t svb, int64_t svh, int64_t svn,
+                       int64_t sob, int64_t soh, int64_t son, float sm_scale, int causal, void *stream);
+
+/*
  * delta[b,h,n] = sum_d O[b,h,n,d] * dO[b,h,n,d], accumulated in fp32.
  * Replaces the launch of _bwd_preprocess_kernel (quant_flash_attn.py:87-101, :217-223).
  * qfa_attn_bwd computes delta inside its own staging pass; this entry point is for callers that

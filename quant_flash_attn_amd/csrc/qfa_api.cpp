@@ -117,6 +117,23 @@ int qfa_attn_fwd(const int8_t *qc, const float *sq, const int8_t *zq, const int3
   return launch_fwd(a, (hipStream_t)stream);
 }
 
+int qfa_bench_qk_stage(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,
+                       const float *sk, const int8_t *zk, const int32_t *rk, const void *v, void *o, float *lse,
+                       int io_dtype, int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D, int64_t sqb, int64_t sqh,
+                       int64_t sqn, int64_t skb, int64_t skh, int64_t skn, int64_t svb, int64_t svh, int64_t svn,
+                       int64_t sob, int64_t soh, int64_t son, float sm_scale, int causal, void *stream) {
+  AttnArgs a;
+  memset(&a, 0, sizeof(a));
+  a.qc = qc; a.sq = sq; a.zq = zq; a.rq = rq; a.kc = kc; a.sk = sk; a.zk = zk; a.rk = rk;
+  a.v = v; a.o = o; a.lse = lse; a.io_dtype = io_dtype;
+  a.B = B; a.H = H; a.Nq = Nq; a.Nk = Nk; a.D = D;
+  a.sqb = sqb; a.sqh = sqh; a.sqn = sqn; a.skb = skb; a.skh = skh; a.skn = skn;
+  a.svb = svb; a.svh = svh; a.svn = svn; a.sob = sob; a.soh = soh; a.son = son;
+  a.sm_scale = sm_scale; a.causal = causal;
+  if (int e = check_attn_common("bench_qk_stage", a)) return e;
+  return launch_fwd(a, (hipStream_t)stream, true);
+}
+
 int qfa_bwd_delta(const void *o, const void *dout, float *delta, int io_dtype, int64_t B, int64_t H, int64_t N,
                   int D, int64_t sob, int64_t soh, int64_t son, int64_t sdb, int64_t sdh, int64_t sdn,
                   void *stream) {

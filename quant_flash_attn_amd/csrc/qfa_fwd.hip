@@ -75,7 +75,11 @@ template <typename T> __device__ __forceinline__ unsigned base128_pair(int n) {
   return pack2<T>((float)(hi * 128), (float)lo);
 }
 
-template <typename T, int D, bool CAUSAL>
+// QK_ONLY is the measurement variant of the same kernel: identical loads, INT8 product, zero-point
+// correction, scaling and running maximum, with the exponentials and the P.V product compiled out
+// (it writes the scaled row maximum where the LSE would go and leaves O untouched).  It exists to
+// time the QK^T stage by itself against the INT8 MFMA peak.
+template <typename T, int D, bool CAUSAL, bool QK_ONLY = false>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
   typedef FwdSmem<D> SM;
   constexpr int KS = D / 32;   // int8 k-steps of 32
@@ -268,6 +272,13 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
   };
   // p = exp2(a_i*u - a_i*m_ref), packed; row sum; O^T += V^T . P^T for the 32 keys of block nb
   auto exp_pv = [&](int vbuf, int nb, const float (&u)[16]) {
+    if (QK_ONLY) {   // keep the scores alive without exponentials or MFMAs
+      float s = 0.f;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s = fmaxf(s, u[v]);
+      l_run = fmaxf(l_run, s);
+      return;
+    }
     const unsigned char *vt_ = smem + SM::OFF_V + vbuf * SM::V_BYTES;
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh) {
@@ -358,6 +369,10 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
   }
 
   // ---- epilogue: normalise, store O (lane holds 4 consecutive d per register quad) and LSE
+  if (QK_ONLY) {
+    if (qi < a.Nq && g == 0) a.lse[tq0 + qi] = a_i * fmaxf(m_ref, l_run);
+    return;
+  }
   const float l_tot = l_run + swap32_f(l_run);
   const float inv = 1.0f / l_tot;
   if (qi < a.Nq) {
@@ -375,7 +390,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
   }
 }
 
-template <typename T, int D> static int launch_fwd_td(const AttnArgs &x, hipStream_t st) {
+template <typename T, int D> static int launch_fwd_td(const AttnArgs &x, hipStream_t st, bool qk_only) {
   FwdArgs a;
   a.qc = x.qc; a.sq = x.sq; a.zq = x.zq; a.rq = x.rq;
   a.kc = x.kc; a.sk = x.sk; a.zk = x.zk; a.rk = x.rk;
@@ -390,18 +405,23 @@ template <typename T, int D> static int launch_fwd_td(const AttnArgs &x, hipStre
   a.total_blocks = (int)total;
   a.blocks_per_xcd = (a.total_blocks + 7) / 8;
   const dim3 grid((unsigned)(a.blocks_per_xcd * 8)), block(256);
-  if (x.causal) fwd_kernel<T, D, true><<<grid, block, 0, st>>>(a);
-  else fwd_kernel<T, D, false><<<grid, block, 0, st>>>(a);
+  if (qk_only) {
+    if (x.causal) fwd_kernel<T, D, true, true><<<grid, block, 0, st>>>(a);
+    else fwd_kernel<T, D, false, true><<<grid, block, 0, st>>>(a);
+  } else {
+    if (x.causal) fwd_kernel<T, D, true><<<grid, block, 0, st>>>(a);
+    else fwd_kernel<T, D, false><<<grid, block, 0, st>>>(a);
+  }
   return check_launch("qfa_attn_fwd");
 }
 
-int launch_fwd(const AttnArgs &x, hipStream_t st) {
+int launch_fwd(const AttnArgs &x, hipStream_t st, bool qk_only) {
   if (x.io_dtype == QFA_BF16) {
-    if (x.D == 128) return launch_fwd_td<__bf16, 128>(x, st);
-    if (x.D == 64) return launch_fwd_td<__bf16, 64>(x, st);
+    if (x.D == 128) return launch_fwd_td<__bf16, 128>(x, st, qk_only);
+    if (x.D == 64) return launch_fwd_td<__bf16, 64>(x, st, qk_only);
   } else if (x.io_dtype == QFA_F16) {
-    if (x.D == 128) return launch_fwd_td<_Float16, 128>(x, st);
-    if (x.D == 64) return launch_fwd_td<_Float16, 64>(x, st);
+    if (x.D == 128) return launch_fwd_td<_Float16, 128>(x, st, qk_only);
+    if (x.D == 64) return launch_fwd_td<_Float16, 64>(x, st, qk_only);
   } else {
     return set_error(QFA_EINVAL, "attn_fwd: io_dtype must be QFA_BF16 or QFA_F16");
   }

@@ -35,7 +35,7 @@ struct AttnArgs {
   int io_dtype;
 };
 
-int launch_fwd(const AttnArgs &a, hipStream_t st);
+int launch_fwd(const AttnArgs &a, hipStream_t st, bool qk_only = false);
 int launch_delta(const void *o, const void *dout, float *delta, int io_dtype, int64_t B, int64_t H, int64_t N, int D,
                  int64_t sob, int64_t soh, int64_t son, int64_t sdb, int64_t sdh, int64_t sdn, hipStream_t st);
 int launch_bwd(const AttnArgs &a, hipStream_t st);

@@ -50,7 +50,7 @@ def _unpack(qt: QuantizedTokens, name: str):
 
 
 def attn_fwd_quantized(qq: QuantizedTokens, kq: QuantizedTokens, v: torch.Tensor, causal: bool,
-                       sm_scale: float) -> Tuple[torch.Tensor, torch.Tensor]:
+                       sm_scale: float, _entry: str = "qfa_attn_fwd") -> Tuple[torch.Tensor, torch.Tensor]:
     """O, LSE = attention(dequant(qq), dequant(kq), v).  v and O are bf16 or fp16 [B,H,N,D];
     LSE is fp32 [B,H,Nq] (natural log, as quant_flash_attn.py:79)."""
     if v.dtype not in _IO_DTYPES:
@@ -66,7 +66,7 @@ def attn_fwd_quantized(qq: QuantizedTokens, kq: QuantizedTokens, v: torch.Tensor
     o = torch.empty((B, H, Nq, D), dtype=v.dtype, device=v.device)
     lse = torch.empty((B, H, Nq), dtype=torch.float32, device=v.device)
     with torch.cuda.device(v.device):
-        code = _lib.lib().qfa_attn_fwd(
+        code = getattr(_lib.lib(), _entry)(     # "qfa_bench_qk_stage" is the QK^T-only timing variant
             qc.data_ptr(), sq.data_ptr(), zq.data_ptr(), rq.data_ptr(),
             kc.data_ptr(), sk.data_ptr(), zk.data_ptr(), rk.data_ptr(),
             v.data_ptr(), o.data_ptr(), lse.data_ptr(), _lib.DTYPE_CODE[v.dtype],
@@ -74,7 +74,7 @@ def attn_fwd_quantized(qq: QuantizedTokens, kq: QuantizedTokens, v: torch.Tensor
             qc.stride(0), qc.stride(1), qc.stride(2), kc.stride(0), kc.stride(1), kc.stride(2),
             v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1), o.stride(2),
             float(sm_scale), int(bool(causal)), _lib.stream_of(v))
-    _lib.check(code, "qfa_attn_fwd")
+    _lib.check(code, _entry)
     return o, lse
 
 
