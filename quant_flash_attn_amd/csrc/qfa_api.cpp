@@ -97,6 +97,9 @@ static int check_attn_common(const char *who, const AttnArgs &a) {
   if (!strides_ok(a.sqb, a.sqh, a.sqn, a.D, 1) || !strides_ok(a.skb, a.skh, a.skn, a.D, 1) ||
       !strides_ok(a.svb, a.svh, a.svn, a.D, 2) || !strides_ok(a.sob, a.soh, a.son, a.D, 2))
     return set_error(QFA_EINVAL, "%s: strides must be positive multiples of 16 bytes, token stride >= D", who);
+  // offsets inside a 64-token tile are formed in 31 bits
+  if (a.skn >= (1 << 23) || a.svn >= (1 << 23) || a.sqn >= (1 << 23))
+    return set_error(QFA_EUNSUPPORTED, "%s: token strides of 2^23 elements or more are not supported", who);
   return 0;
 }
 

@@ -92,6 +92,16 @@ template <int CTRL> __device__ __forceinline__ int dpp_i(int x) {
 // value held by lane (l ^ 32)
 __device__ __forceinline__ float swap32_f(float x) { return __shfl_xor(x, 32, 64); }
 
+// max of x over the lane pair (l, l ^ 32).  v_permlane32_swap exchanges the upper half of its first
+// register with the lower half of its second; fed two copies of x it leaves {lo,lo} and {hi,hi}.
+// (Inline asm: the builtin's second result is not usable with this compiler; the instruction needs
+// two wait states after a vector write of its operands.)
+__device__ __forceinline__ float max_across_halves(float x) {
+  float lo = x, hi = x;
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(lo), "+v"(hi));
+  return fmaxf(lo, hi);
+}
+
 // ---- direct global -> LDS tile copies -------------------------------------------------------------
 // global_load_lds_dwordx4 writes lane l's 16 bytes to LDS[wave-uniform base + 16*l], so a tile lands
 // in LDS as dense rows without padding.  Bank conflicts are avoided by an XOR swizzle applied on the
@@ -106,14 +116,30 @@ template <int ROW_BYTES> struct Swz {
   static __device__ __forceinline__ int off(int r, int c) { return r * ROW_BYTES + ((c ^ swz(r)) << 4); }
 };
 
+// Raw buffer descriptor over [p, p + bytes): loads through it take a per-lane 32-bit offset plus a
+// scalar offset (no 64-bit address arithmetic on the vector pipe) and return zero out of range.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
+}
+
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
+// Swizzle for tiles of 16-bit elements that are read back with ds_read_b64_tr_b16: there the 32 lanes
+// of one k-group read 64 contiguous bytes from each of 4 consecutive rows, so the XOR moves whole
+// 64-byte quarters of the 256-byte bank line: position q of row r holds chunk q ^ swz(r).
+template <int ROW_BYTES> struct SwzQuad {
+  static constexpr int CPR = ROW_BYTES / 16;
+  static constexpr int RPL = ROW_BYTES >= 256 ? 1 : 256 / ROW_BYTES;   // rows per 256-byte line
+  static constexpr int QPR = ROW_BYTES / 64;                             // 64-byte quarters per row
+  static __device__ __forceinline__ int swz(int row) { return 4 * ((row / RPL) % QPR); }
+};
+
 // rows [row0, row0+ROWS) (clamped to row_max) of a row-major global array -> swizzled LDS tile; NT threads
-template <int ROW_BYTES, int ROWS, int NT>
+template <int ROW_BYTES, int ROWS, int NT, typename S = Swz<ROW_BYTES>>
 __device__ __forceinline__ void dma_rows(const unsigned char *g, int64_t gstride, int row0, int row_max,
                                          unsigned char *lds, int tid) {
-  typedef Swz<ROW_BYTES> S;
   constexpr int TOTAL = ROWS * S::CPR;
 #pragma unroll
   for (int i = 0; i < (TOTAL + NT - 1) / NT; ++i) {
@@ -143,6 +169,33 @@ __device__ __forceinline__ void dma_wait() { __builtin_amdgcn_s_waitcnt(0x0f70);
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
 // global access, including direct-to-LDS loads issued for a LATER tile, which would serialise the
 // prefetch; this one leaves them in flight (pair it with dma_wait() where a tile must have landed).
+// ds_read_b64_tr_b16: inside each group of 16 lanes, lane i receives element i%4 of the four 8-byte
+// rows addressed by lanes (i%16)/4, +4, +8, +12 of its group -- a 16-bit transpose on the way out of LDS.
+__device__ __forceinline__ u32x2 lds_read_tr16(const unsigned char *p) {
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p));
+}
+// The same read issued behind the compiler's back, with an explicit wait.  The compiler makes every
+// ds_read_b64_tr_b16 it knows of wait for ALL outstanding direct-to-LDS loads (it cannot tell which
+// buffer they fill), which would expose the latency of the next tile's copy once per tile.  The asm
+// form is invisible to that bookkeeping, so the result must not be used before one of the waits
+// below, which take the loaded registers as operands to keep their consumers behind them.
+// LDS operations return in order: lgkmcnt(N) guarantees everything but the last N issued is there.
+__device__ __forceinline__ unsigned lds_addr(const void *p) { return (unsigned)(size_t)(lptr_t)p; }
+template <int OFF> __device__ __forceinline__ u32x2 lds_read_tr16_async(unsigned addr) {
+  u32x2 r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+template <int N> __device__ __forceinline__ void lds_wait_async(u32x2 (&r)[8]) {
+  asm volatile("s_waitcnt lgkmcnt(%8)"
+               : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7])
+               : "n"(N)
+               : "memory");
+}
+template <int N> __device__ __forceinline__ void lds_wait_async(u32x2 (&r)[4]) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]) : "n"(N) : "memory");
+}
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 }  // namespace qfa

@@ -2,8 +2,10 @@
 // INT8 codes (scale, zero point, row sum per token).  gfx950, wave64.
 //
 // Work split.  One workgroup = 4 waves = 128 query rows of one (batch, head); each wave owns
-// 32 queries.  K (3 buffers) and V (2 buffers) stream through LDS in tiles of 64 keys: K and the
-// per-key constants are resident one tile ahead of V because the score product runs ahead.
+// 32 queries.  K (3 buffers) and V (2 buffers) stream through LDS in tiles of 64 keys, copied by
+// direct global->LDS loads (no staging registers, no address or repacking work on the vector
+// pipe); K and the per-key constants are resident one tile ahead of V because the score product
+// runs ahead.
 //
 // Score tile.  Each wave computes S^T = Kc . Qc^T with v_mfma_i32_32x32x32_i8: the K rows come
 // from LDS (A operand), the wave's 32 queries stay in registers for the whole kernel (B operand).
@@ -30,9 +32,11 @@
 //    of block b+2 and the convert/correct/scale/max of block b+1 are independent of each other,
 //    so MFMA and VALU instructions interleave; diagonal and ragged tiles run a simple masked loop.
 //
-// V is transposed on its way into LDS (Vt[d][key]) so a lane reads its 8 keys of one d as one
-// 16-byte LDS load; keys are stored in the permuted order in which the S^T accumulator layout
-// hands out P, so no shuffle is needed between the two products.
+// V lies in LDS as it does in memory ([key][d] rows, 64-byte quarters XOR-swizzled against bank
+// conflicts) and is transposed on the way out: ds_read_b64_tr_b16 hands lane (d, k-group) four
+// consecutive keys of its d, and two such reads give exactly the 8 keys whose probabilities the
+// S^T accumulator layout left in that k-group's registers, so no shuffle is needed between the two
+// products.
 #include <type_traits>
 
 #include "qfa_device.h"
@@ -58,10 +62,10 @@ constexpr int FWD_BN = 64;
 constexpr float FWD_RESCALE_THRESHOLD = 8.0f;   // log2 units the running max may lag behind
 
 template <int D> struct FwdSmem {
-  static constexpr int KSTR = D + 16;            // bytes per K row (+16: conflict-free 16-byte reads)
-  static constexpr int VSTR = (FWD_BN + 8) * 2;  // bytes per Vt row
+  static constexpr int KSTR = D;                 // bytes per K row (dense, chunks swizzled: Swz<D>)
+  static constexpr int VSTR = 2 * D;             // bytes per V row (dense, quarters swizzled: SwzQuad<2D>)
   static constexpr int K_BYTES = FWD_BN * KSTR;
-  static constexpr int V_BYTES = D * VSTR;
+  static constexpr int V_BYTES = FWD_BN * VSTR;
   static constexpr int C_BYTES = FWD_BN * 4 + FWD_BN * 8;  // key scale; correction digits (2 dwords/key)
   static constexpr int OFF_K = 0;                     // 3 buffers
   static constexpr int OFF_V = 3 * K_BYTES;           // 2 buffers
@@ -84,7 +88,6 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
   typedef FwdSmem<D> SM;
   constexpr int KS = D / 32;   // int8 k-steps of 32
   constexpr int DB = D / 32;   // 32-row blocks of O^T
-  constexpr int KCH = (FWD_BN * D / 16) / 256;   // 16-byte K chunks per thread (2 for D=128, 1 for D=64)
   __shared__ __attribute__((aligned(16))) unsigned char smem[SM::TOTAL];
 
   // ---- block -> (batch*head, query block); consecutive ids of one XCD share a head's K/V in its L2
@@ -134,41 +137,58 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
   if (CAUSAL) kv_end = min(a.Nk, m0 + FWD_BM);
   const int ntiles = (kv_end + FWD_BN - 1) / FWD_BN;
 
-  // ---- loader roles
-  const int v_kv4 = tid % 16;   // group of 4 consecutive keys
-  const int v_dc = tid / 16;    // chunk of 8 consecutive d
-  const bool v_active = v_dc < D / 8;
-  const int v_pos = 32 * (v_kv4 / 8) + 16 * ((v_kv4 / 4) % 2) + 8 * (v_kv4 % 2) + 4 * ((v_kv4 / 2) % 2);
-
-  u32x4 kreg[KCH];
-  u32x4 vreg[4];
+  // ---- tile copies: K and V by direct loads, the per-key constants through registers
+  typedef Swz<D> KSW;
+  typedef SwzQuad<2 * D> VSW;
   float c_sk;
   int c_rk, c_zk;
 
-  auto load_k = [&](int t) {
-    const int j0 = t * FWD_BN;
+  // Per-thread byte offsets of its 16-byte chunks inside a full tile (row * stride + swizzled chunk);
+  // the tile's first row goes into the wave-uniform base, so a full tile costs no address arithmetic
+  // on the vector pipe.  Ragged tiles (rows clamped to the last key) take the generic path.
+  constexpr int KCH = FWD_BN * (D / 16) / 256;        // K chunks per thread
+  constexpr int VCH = FWD_BN * (2 * D / 16) / 256;    // V chunks per thread
+  unsigned koff[KCH], voff[VCH];
 #pragma unroll
-    for (int i = 0; i < KCH; ++i) {
-      const int c = tid + 256 * i;
-      const int row = c / (D / 16), col = c % (D / 16);
-      const int j = min(j0 + row, a.Nk - 1);
-      kreg[i] = *reinterpret_cast<const u32x4 *>(kc_bh + (int64_t)j * a.skn + col * 16);
-    }
+  for (int i = 0; i < KCH; ++i) {
+    const int p = tid + 256 * i, row = p / KSW::CPR, pos = p % KSW::CPR;
+    koff[i] = (unsigned)row * (unsigned)a.skn + (unsigned)((pos ^ KSW::swz(row)) << 4);
+  }
+#pragma unroll
+  for (int i = 0; i < VCH; ++i) {
+    const int p = tid + 256 * i, row = p / VSW::CPR, pos = p % VSW::CPR;
+    voff[i] = (unsigned)row * (unsigned)(a.svn * sizeof(T)) + (unsigned)((pos ^ VSW::swz(row)) << 4);
+  }
+
+  // Full tiles are copied through buffer descriptors rebased to the tile's first row (scalar
+  // arithmetic), so a copy costs one instruction per 16-byte chunk and thread; the per-key constant
+  // vectors are read the same way, with exact bounds (keys past the end read as zero and are masked).
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const rsrc_t rs_sk = make_rsrc(a.sk + tk0, (unsigned)a.Nk * 4u);
+  const rsrc_t rs_rk = make_rsrc(a.rk + tk0, (unsigned)a.Nk * 4u);
+  const rsrc_t rs_zk = make_rsrc(a.zk + tk0, (unsigned)a.Nk);
+  auto load_kc = [&](int t) {   // per-key constants of tile t -> registers
     if (tid < FWD_BN) {
-      const int j = min(j0 + tid, a.Nk - 1);
-      c_sk = a.sk[tk0 + j];
-      c_rk = a.rk[tk0 + j];
-      c_zk = (int)a.zk[tk0 + j];
+      c_sk = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_sk, tid * 4, t * FWD_BN * 4, 0));
+      c_rk = __builtin_amdgcn_raw_buffer_load_b32(rs_rk, tid * 4, t * FWD_BN * 4, 0);
+      c_zk = (int)(signed char)__builtin_amdgcn_raw_buffer_load_b8(rs_zk, tid, t * FWD_BN, 0);
     }
   };
-  auto store_k = [&](int buf) {
-    unsigned char *base = smem + SM::OFF_K + buf * SM::K_BYTES;
+  auto load_k = [&](int t, int buf) {
+    const int j0 = t * FWD_BN;
+    unsigned char *dst = smem + SM::OFF_K + buf * SM::K_BYTES;
+    if (j0 + FWD_BN <= a.Nk) {
+      const rsrc_t rs = make_rsrc(reinterpret_cast<const unsigned char *>(kc_bh) + (int64_t)j0 * a.skn, 0x7fffffffu);
 #pragma unroll
-    for (int i = 0; i < KCH; ++i) {
-      const int c = tid + 256 * i;
-      const int row = c / (D / 16), col = c % (D / 16);
-      *reinterpret_cast<u32x4 *>(base + row * SM::KSTR + col * 16) = kreg[i];
+      for (int i = 0; i < KCH; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lptr_t)(dst + (wave_u * 64 + 256 * i) * 16), 16, (int)koff[i], 0, 0,
+                                                 0);
+    } else {
+      dma_rows<D, FWD_BN, 256, KSW>(reinterpret_cast<const unsigned char *>(kc_bh), a.skn, j0, a.Nk - 1, dst, tid);
     }
+    load_kc(t);
+  };
+  auto store_k = [&](int buf) {
     if (tid < FWD_BN) {
       unsigned char *cb = smem + SM::OFF_C + buf * SM::C_BYTES;
       reinterpret_cast<float *>(cb)[tid] = c_sk;
@@ -180,32 +200,23 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
   };
   auto load_v = [&](int t) {
     const int j0 = t * FWD_BN;
-    if (v_active) {
+    unsigned char *dst = smem + SM::OFF_V + (t & 1) * SM::V_BYTES;
+    const int64_t vstride = a.svn * (int64_t)sizeof(T);
+    if (j0 + FWD_BN <= a.Nk) {
+      const rsrc_t rs = make_rsrc(reinterpret_cast<const unsigned char *>(v_bh) + (int64_t)j0 * vstride, 0x7fffffffu);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int j = min(j0 + 4 * v_kv4 + r, a.Nk - 1);
-        vreg[r] = *reinterpret_cast<const u32x4 *>(v_bh + (int64_t)j * a.svn + v_dc * 8);
-      }
+      for (int i = 0; i < VCH; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lptr_t)(dst + (wave_u * 64 + 256 * i) * 16), 16, (int)voff[i], 0, 0,
+                                                 0);
+    } else {
+      dma_rows<2 * D, FWD_BN, 256, VSW>(reinterpret_cast<const unsigned char *>(v_bh), vstride, j0, a.Nk - 1, dst, tid);
     }
   };
-  auto store_v = [&](int buf) {
-    if (v_active) {
-      unsigned char *vt = smem + SM::OFF_V + buf * SM::V_BYTES;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {   // d = 8*v_dc + e: gather the 4 keys of that d
-        const int w = e / 2;
-        u32x2 o;
-        if (e % 2 == 0) {
-          o[0] = (vreg[0][w] & 0xffffu) | (vreg[1][w] << 16);
-          o[1] = (vreg[2][w] & 0xffffu) | (vreg[3][w] << 16);
-        } else {
-          o[0] = (vreg[0][w] >> 16) | (vreg[1][w] & 0xffff0000u);
-          o[1] = (vreg[2][w] >> 16) | (vreg[3][w] & 0xffff0000u);
-        }
-        *reinterpret_cast<u32x2 *>(vt + (v_dc * 8 + e) * SM::VSTR + v_pos * 2) = o;
-      }
-    }
-  };
+  // this lane's read offsets inside a tile (the swizzle terms only depend on the lane)
+  const int k_swz = KSW::swz(lr);                                        // rows 32*nb + lr
+  const int v_row = (lane % 16) / 4;                                     // source row of the transposing read
+  const int v_off = v_row * SM::VSTR + ((VSW::swz(v_row) + 2 * ((lane / 16) % 2) + (lane % 4) / 2) << 4) +
+                    8 * (lane % 2);                                      // XOR with 64*db selects the d block
   // S^T block nb (32 keys) of the tile held in K buffer `buf`, for this wave's 32 queries
   auto qk_block = [&](int buf, int nb, i32x16 &s) {
     const unsigned char *ks_ = smem + SM::OFF_K + buf * SM::K_BYTES;
@@ -213,7 +224,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
     for (int v = 0; v < 16; ++v) s[v] = 0;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const i32x4 kf = *reinterpret_cast<const i32x4 *>(ks_ + (32 * nb + lr) * SM::KSTR + ks * 32 + g * 16);
+      const i32x4 kf =
+          *reinterpret_cast<const i32x4 *>(ks_ + (32 * nb + lr) * SM::KSTR + (((2 * ks + g) ^ k_swz) << 4));
       s = mfma_i8(kf, qf[ks], s);
     }
   };
@@ -254,7 +266,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
         mt = fmaxf(mt, uu);
       }
     }
-    return fmaxf(mt, swap32_f(mt));
+    return max_across_halves(mt);
   };
   // move the reference maximum only when some row of the wave outgrew it by > 2^threshold
   auto rescale_if_needed = [&](float mt) {
@@ -292,22 +304,24 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
       }
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const u32x4 vf =
-            *reinterpret_cast<const u32x4 *>(vt_ + (32 * db + lr) * SM::VSTR + (32 * nb + 16 * hh + 8 * g) * 2);
+        // keys 32nb + 16hh + 4g + {0..3} and those + 8: the order in which pf holds the probabilities
+        const unsigned char *vp = vt_ + (32 * nb + 16 * hh + 4 * g) * SM::VSTR + (v_off ^ (64 * db));
+        const u32x2 v0 = lds_read_tr16(vp), v1 = lds_read_tr16(vp + 8 * SM::VSTR);
+        const u32x4 vf = {v0[0], v0[1], v1[0], v1[1]};
         oacc[db] = mfma_16b<T>(vf, pf, oacc[db]);
       }
     }
   };
 
   // ---- prologue: K(0), K(1) (with their constants) and V(0) resident
-  load_k(0);
+  load_k(0, 0);
   load_v(0);
   store_k(0);
-  store_v(0);
   if (ntiles > 1) {
-    load_k(1);
+    load_k(1, 1);
     store_k(1);
   }
+  dma_wait();
   __syncthreads();
 
   // tiles [0, t_hot) contain no masked score for this wave (wave-uniform)
@@ -317,39 +331,139 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
 
   int kb_cur = 0, kb_nxt = 1, kb_free = 2;   // K/constant buffers of tile t, t+1, and the one to refill
   int t = 0;
-  {
-    // ---- pipelined loop over unmasked tiles.  Entering tile t: u_a = prepared block 2t,
-    // s_y = raw S of block 2t+1; the reference maximum already covers block 2t.
-    float u_a[16], u_b[16];
-    i32x16 s_x, s_y;
-    if (t_hot > 0) {
-      qk_block(0, 0, s_x);
-      qk_block(0, 1, s_y);
-      rescale_if_needed(prep(0, 0, s_x, u_a, 0, std::false_type{}));
+  if (t_hot > 0) {
+    // ---- pipelined loop over unmasked tiles, one straight-line body per 32-key block b:
+    //   exp2/pack and P.V of block b | INT8 product of block b+1 | convert/correct/scale/max of b+1,
+    // with every LDS operand requested a phase (or a body) before the MFMA that consumes it.  The
+    // phases are fenced so that the requests stay where they are; inside a phase MFMA and VALU
+    // instructions are independent and interleave.
+    // Carried between bodies: u = prepared scores of block b, kf = K fragments of block b+1.
+    float u[16];
+    i32x4 kf[KS];
+    auto k_frags = [&](int buf, int nb) {
+      const unsigned char *ks_ = smem + SM::OFF_K + buf * SM::K_BYTES;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        kf[ks] = *reinterpret_cast<const i32x4 *>(ks_ + (32 * nb + lr) * SM::KSTR + (((2 * ks + g) ^ k_swz) << 4));
+    };
+    // V fragments of keys 32nb + 16hh + 4g + {0..3} and those + 8 (the order in which pf holds the
+    // probabilities), requested without the compiler's knowledge: pair every call with lds_wait_async
+    auto v_frags = [&](int vbuf, auto nb_tag, auto hh_tag, u32x2 (&vr)[2 * DB]) {
+      constexpr int ROW0 = (32 * decltype(nb_tag)::value + 16 * decltype(hh_tag)::value) * SM::VSTR;
+      const unsigned base = lds_addr(smem + SM::OFF_V) + vbuf * SM::V_BYTES + 4 * g * SM::VSTR;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const unsigned ad = base + (v_off ^ (64 * db));
+        vr[2 * db] = lds_read_tr16_async<ROW0>(ad);
+        vr[2 * db + 1] = lds_read_tr16_async<ROW0 + 8 * SM::VSTR>(ad);
+      }
+    };
+    auto exp_half = [&](int hh, u32x4 &pf) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, u[8 * hh + 2 * e], nm));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, u[8 * hh + 2 * e + 1], nm));
+        pf[e] = pack2<T>(p0, p1);
+      }
+    };
+    // one body: V block (vbuf, nb); scores of the next block from kf; its constants in (cbuf, cnb);
+    // then kf is refilled from K block (kbuf, knb).  `count_max`: whether the next block's maximum
+    // may move the reference (false when that block belongs to a masked tile and is recomputed there).
+    auto body = [&](int vbuf, auto nb_tag, int cbuf, int cnb, int kbuf, int knb, bool count_max) {
+      static_assert(DB == 4 || DB == 2, "fragment arrays are sized for head_dim 128 or 64");
+      u32x2 vr0[2 * DB], vr1[2 * DB];
+      u32x4 pf0, pf1;
+      i32x16 s;
+      const auto NB = nb_tag;
+      if (!QK_ONLY) v_frags(vbuf, NB, std::integral_constant<int, 0>{}, vr0);
+      __builtin_amdgcn_sched_barrier(0);
+      // INT8 product of block b+1 under the exponentials of the first 16 keys of block b
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s[v] = 0;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) s = mfma_i8(kf[ks], qf[ks], s);
+      if (!QK_ONLY) exp_half(0, pf0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (!QK_ONLY) {
+        v_frags(vbuf, NB, std::integral_constant<int, 1>{}, vr1);
+        lds_wait_async<2 * DB>(vr0);   // the 2*DB requests just made may still be in flight
+      }
+      const unsigned char *cb = smem + SM::OFF_C + cbuf * SM::C_BYTES;
+      f32x4 sk4[4];
+#pragma unroll
+      for (int aa = 0; aa < 4; ++aa)
+        sk4[aa] = *reinterpret_cast<const f32x4 *>(cb + (32 * cnb + 8 * aa + 4 * g) * 4);
+      const u32x4 corr_k = {reinterpret_cast<const unsigned *>(cb + FWD_BN * 4)[2 * (32 * cnb + lr) + g], 0u, 0u, 0u};
+      __builtin_amdgcn_sched_barrier(0);
+      if (!QK_ONLY) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+          oacc[db] = mfma_16b<T>(u32x4{vr0[2 * db][0], vr0[2 * db][1], vr0[2 * db + 1][0], vr0[2 * db + 1][1]}, pf0,
+                                 oacc[db]);
+        exp_half(1, pf1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (!QK_ONLY) lds_wait_async<0>(vr1);   // everything requested so far was requested a phase ago
+      k_frags(kbuf, knb);
+      __builtin_amdgcn_sched_barrier(0);
+      f32x16 f;
+      if (!QK_ONLY) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+          oacc[db] = mfma_16b<T>(u32x4{vr1[2 * db][0], vr1[2 * db][1], vr1[2 * db + 1][0], vr1[2 * db + 1][1]}, pf1,
+                                 oacc[db]);
+      } else {
+        float sm = 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sm = fmaxf(sm, u[v]);
+        l_run = fmaxf(l_run, sm);
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
+      __builtin_amdgcn_sched_barrier(0);
+      f = mfma_16b<T>(corr_k, corr_q, f);
+      if (!QK_ONLY) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) l_run = dot2_ones<T>(pf0[e], l_run);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) l_run = dot2_ones<T>(pf1[e], l_run);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      float mt = -INFINITY;
+#pragma unroll
+      for (int aa = 0; aa < 4; ++aa)
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb) {
+          u[4 * aa + bb] = f[4 * aa + bb] * sk4[aa][bb];
+          mt = fmaxf(mt, u[4 * aa + bb]);
+        }
+      mt = max_across_halves(mt);
+      rescale_if_needed(count_max ? mt : -INFINITY);
+    };
+
+    {   // block 0 prepared, fragments of block 1 in flight
+      i32x16 s0;
+      qk_block(0, 0, s0);
+      float u0[16];
+      rescale_if_needed(prep(0, 0, s0, u0, 0, std::false_type{}));
+#pragma unroll
+      for (int v = 0; v < 16; ++v) u[v] = u0[v];
+      k_frags(0, 1);
     }
     for (; t < t_hot; ++t) {
-      if (t + 2 < ntiles) load_k(t + 2);
+      if (t + 2 < ntiles) load_k(t + 2, kb_free);
       if (t + 1 < ntiles) load_v(t + 1);
-      // block 2t: consume u_a; raw S(2t+2) -> s_x; prepare block 2t+1 from s_y
-      qk_block(kb_nxt, 0, s_x);
-      exp_pv(t & 1, 0, u_a);
-      rescale_if_needed(prep(kb_cur, 1, s_y, u_b, 0, std::false_type{}));
-      // block 2t+1: consume u_b; raw S(2t+3) -> s_y; prepare block 2t+2 from s_x (only a
-      // candidate maximum if that block belongs to the unmasked range)
-      qk_block(kb_nxt, 1, s_y);
-      exp_pv(t & 1, 1, u_b);
-      const float mt = prep(kb_nxt, 0, s_x, u_a, 0, std::false_type{});
-      rescale_if_needed(t + 1 < t_hot ? mt : -INFINITY);
-
+      body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, true);
+      body(t & 1, std::integral_constant<int, 1>{}, kb_nxt, 0, kb_nxt, 1, t + 1 < t_hot);
       if (t + 2 < ntiles) store_k(kb_free);
-      if (t + 1 < ntiles) store_v((t + 1) & 1);
       const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
+      dma_wait();
       __syncthreads();
     }
   }
   // ---- masked tiles (diagonal, ragged end): one block at a time, nothing carried between blocks
   for (; t < ntiles; ++t) {
-    if (t + 2 < ntiles) load_k(t + 2);
+    if (t + 2 < ntiles) load_k(t + 2, kb_free);
     if (t + 1 < ntiles) load_v(t + 1);
     const int j0 = t * FWD_BN;
 #pragma unroll
@@ -363,8 +477,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
       exp_pv(t & 1, nb, u);
     }
     if (t + 2 < ntiles) store_k(kb_free);
-    if (t + 1 < ntiles) store_v((t + 1) & 1);
     const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
+    dma_wait();
     __syncthreads();
   }
 
