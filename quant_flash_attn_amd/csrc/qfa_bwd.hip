@@ -307,13 +307,28 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(BwdArgs a) {
   if (CAUSAL) kv_end = min(a.Nk, m0 + DQ_BLK);
   const int ntiles = (kv_end + BWD_TILE - 1) / BWD_TILE;
 
+  // full tiles: per-thread offsets computed once, one copy instruction per chunk afterwards
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  TileCopy<D, BWD_TILE, DQ_THREADS> cp_k;
+  TileCopy<2 * D, BWD_TILE, DQ_THREADS> cp_v;
+  TileCopy<BWD_TILE * 2, D, DQ_THREADS> cp_t;
+  TileCopy<WS::CK_BYTES, 1, DQ_THREADS, NoSwz<WS::CK_BYTES>> cp_c;
+  cp_k.init((unsigned)a.skn, tid);
+  cp_v.init((unsigned)a.svn * 2u, tid);
+  cp_t.init(BWD_TILE * 2, tid);
+  cp_c.init(0, tid);
   auto load_tile = [&](int t) {
     unsigned char *base = smem + (t & 1) * BUF;
     const unsigned char *blob = wsk_bh + (int64_t)t * WS::K_BLOB;
-    dma_rows<D, BWD_TILE, DQ_THREADS>(kc_bh, a.skn, t * BWD_TILE, a.Nk - 1, base, tid);
-    dma_rows<2 * D, BWD_TILE, DQ_THREADS>(v_bh, a.svn * 2, t * BWD_TILE, a.Nk - 1, base + OFF_V, tid);
-    dma_rows<BWD_TILE * 2, D, DQ_THREADS>(blob, BWD_TILE * 2, 0, D - 1, base + OFF_T, tid);
-    dma_flat<WS::CK_BYTES, DQ_THREADS>(blob + WS::T_BYTES, base + OFF_C, tid);
+    if ((t + 1) * BWD_TILE <= a.Nk) {
+      cp_k.issue(kc_bh + (int64_t)t * BWD_TILE * a.skn, base, wave_u, tid);
+      cp_v.issue(v_bh + (int64_t)t * BWD_TILE * a.svn * 2, base + OFF_V, wave_u, tid);
+    } else {
+      dma_rows<D, BWD_TILE, DQ_THREADS>(kc_bh, a.skn, t * BWD_TILE, a.Nk - 1, base, tid);
+      dma_rows<2 * D, BWD_TILE, DQ_THREADS>(v_bh, a.svn * 2, t * BWD_TILE, a.Nk - 1, base + OFF_V, tid);
+    }
+    cp_t.issue(blob, base + OFF_T, wave_u, tid);
+    cp_c.issue(blob + WS::T_BYTES, base + OFF_C, wave_u, tid);
   };
 
   f32x16 dqacc[DB];
@@ -476,14 +491,29 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
   const int it0 = CAUSAL ? n0 / BWD_TILE : 0;
   const int ntiles = a.tiles_q;
 
+  // full tiles: per-thread offsets computed once, one copy instruction per chunk afterwards
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  TileCopy<D, BWD_TILE, DKV_THREADS> cp_q;
+  TileCopy<2 * D, BWD_TILE, DKV_THREADS> cp_g;
+  TileCopy<BWD_TILE * 2, D, DKV_THREADS> cp_t;
+  TileCopy<WS::CQ_BYTES, 1, DKV_THREADS, NoSwz<WS::CQ_BYTES>> cp_c;
+  cp_q.init((unsigned)a.sqn, tid);
+  cp_g.init((unsigned)a.sdon * 2u, tid);
+  cp_t.init(BWD_TILE * 2, tid);
+  cp_c.init(0, tid);
   auto load_tile = [&](int t) {
     unsigned char *base = smem + (t & 1) * BUF;
     const unsigned char *blob = wsq_bh + (int64_t)t * WS::Q_BLOB;
-    dma_rows<D, BWD_TILE, DKV_THREADS>(qc_bh, a.sqn, t * BWD_TILE, a.Nq - 1, base, tid);
-    dma_rows<2 * D, BWD_TILE, DKV_THREADS>(do_bh, a.sdon * 2, t * BWD_TILE, a.Nq - 1, base + OFF_DO, tid);
-    dma_rows<BWD_TILE * 2, D, DKV_THREADS>(blob, BWD_TILE * 2, 0, D - 1, base + OFF_DOT, tid);
-    dma_rows<BWD_TILE * 2, D, DKV_THREADS>(blob + WS::T_BYTES, BWD_TILE * 2, 0, D - 1, base + OFF_QT, tid);
-    dma_flat<WS::CQ_BYTES, DKV_THREADS>(blob + 2 * WS::T_BYTES, base + OFF_C, tid);
+    if ((t + 1) * BWD_TILE <= a.Nq) {
+      cp_q.issue(qc_bh + (int64_t)t * BWD_TILE * a.sqn, base, wave_u, tid);
+      cp_g.issue(do_bh + (int64_t)t * BWD_TILE * a.sdon * 2, base + OFF_DO, wave_u, tid);
+    } else {
+      dma_rows<D, BWD_TILE, DKV_THREADS>(qc_bh, a.sqn, t * BWD_TILE, a.Nq - 1, base, tid);
+      dma_rows<2 * D, BWD_TILE, DKV_THREADS>(do_bh, a.sdon * 2, t * BWD_TILE, a.Nq - 1, base + OFF_DO, tid);
+    }
+    cp_t.issue(blob, base + OFF_DOT, wave_u, tid);
+    cp_t.issue(blob + WS::T_BYTES, base + OFF_QT, wave_u, tid);
+    cp_c.issue(blob + 2 * WS::T_BYTES, base + OFF_C, wave_u, tid);
   };
 
   f32x16 oacc[DB];   // dV^T (P role) or dK^T (dS role) for this lane's key

@@ -153,6 +153,35 @@ __device__ __forceinline__ void dma_rows(const unsigned char *g, int64_t gstride
     }
   }
 }
+// The same copy for FULL tiles (no row clamping), with everything per-thread computed once: off[]
+// holds the thread's byte offsets from the tile's first row, and each copy rebases a buffer
+// descriptor to that row with scalar arithmetic, so a tile costs one instruction per chunk and thread.
+template <int ROW_BYTES, int ROWS, int NT, typename S = Swz<ROW_BYTES>> struct TileCopy {
+  static constexpr int TOTAL = ROWS * S::CPR;
+  static constexpr int N = (TOTAL + NT - 1) / NT;
+  unsigned off[N];
+  __device__ __forceinline__ void init(unsigned gstride, int tid) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int p = tid + NT * i, row = p / S::CPR, pos = p % S::CPR;
+      off[i] = (unsigned)row * gstride + (unsigned)((pos ^ S::swz(row)) << 4);
+    }
+  }
+  // tile_base and lds must be wave-uniform; wave_u = wave index held in a scalar register
+  __device__ __forceinline__ void issue(const void *tile_base, unsigned char *lds, int wave_u, int tid) const {
+    const rsrc_t rs = make_rsrc(tile_base, 0x7fffffffu);
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+      if (TOTAL % NT == 0 || tid + NT * i < TOTAL)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lptr_t)(lds + (wave_u * 64 + NT * i) * 16), 16, (int)off[i], 0, 0, 0);
+  }
+};
+// dense swizzle-free layout for TileCopy (contiguous bytes)
+template <int ROW_BYTES> struct NoSwz {
+  static constexpr int CPR = ROW_BYTES / 16;
+  static __device__ __forceinline__ int swz(int) { return 0; }
+};
+
 // BYTES contiguous bytes, copied as they are
 template <int BYTES, int NT>
 __device__ __forceinline__ void dma_flat(const unsigned char *g, unsigned char *lds, int tid) {

@@ -39,45 +39,9 @@
 // products.
 #include <type_traits>
 
-#include "qfa_device.h"
-#include "qfa_host.h"
+#include "qfa_fwd_common.h"
 
 namespace qfa {
-
-struct FwdArgs {
-  const int8_t *qc; const float *sq; const int8_t *zq; const int32_t *rq;
-  const int8_t *kc; const float *sk; const int8_t *zk; const int32_t *rk;
-  const void *v; void *o; float *lse;
-  int64_t H;
-  int Nq, Nk;
-  int64_t sqb, sqh, sqn, skb, skh, skn, svb, svh, svn, sob, soh, son;
-  float sm_scale_log2;   // sm_scale * log2(e)
-  int mblocks;           // ceil(Nq / 128)
-  int total_blocks;      // mblocks * B * H
-  int blocks_per_xcd;    // ceil(total_blocks / 8)
-};
-
-constexpr int FWD_BM = 128;
-constexpr int FWD_BN = 64;
-constexpr float FWD_RESCALE_THRESHOLD = 8.0f;   // log2 units the running max may lag behind
-
-template <int D> struct FwdSmem {
-  static constexpr int KSTR = D;                 // bytes per K row (dense, chunks swizzled: Swz<D>)
-  static constexpr int VSTR = 2 * D;             // bytes per V row (dense, quarters swizzled: SwzQuad<2D>)
-  static constexpr int K_BYTES = FWD_BN * KSTR;
-  static constexpr int V_BYTES = FWD_BN * VSTR;
-  static constexpr int C_BYTES = FWD_BN * 4 + FWD_BN * 8;  // key scale; correction digits (2 dwords/key)
-  static constexpr int OFF_K = 0;                     // 3 buffers
-  static constexpr int OFF_V = 3 * K_BYTES;           // 2 buffers
-  static constexpr int OFF_C = OFF_V + 2 * V_BYTES;   // 3 buffers
-  static constexpr int TOTAL = OFF_C + 3 * C_BYTES;
-};
-
-// integer n in [-32768, 32767] -> (128*floor(n/128), n mod 128) as a packed pair of 16-bit floats
-template <typename T> __device__ __forceinline__ unsigned base128_pair(int n) {
-  const int hi = n >> 7, lo = n & 127;
-  return pack2<T>((float)(hi * 128), (float)lo);
-}
 
 // QK_ONLY is the measurement variant of the same kernel: identical loads, INT8 product, zero-point
 // correction, scaling and running maximum, with the exponentials and the P.V product compiled out
