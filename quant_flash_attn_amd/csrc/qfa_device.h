@@ -167,6 +167,11 @@ template <int ROW_BYTES, int ROWS, int NT, typename S = Swz<ROW_BYTES>> struct T
       off[i] = (unsigned)row * gstride + (unsigned)((pos ^ S::swz(row)) << 4);
     }
   }
+  // one chunk (index i < N) of a copy whose descriptor the caller made with make_rsrc(tile_base, ...)
+  __device__ __forceinline__ void issue_one(rsrc_t rs, unsigned char *lds, int wave_u, int tid, int i) const {
+    if (TOTAL % NT == 0 || tid + NT * i < TOTAL)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lptr_t)(lds + (wave_u * 64 + NT * i) * 16), 16, (int)off[i], 0, 0, 0);
+  }
   // tile_base and lds must be wave-uniform; wave_u = wave index held in a scalar register
   __device__ __forceinline__ void issue(const void *tile_base, unsigned char *lds, int wave_u, int tid) const {
     const rsrc_t rs = make_rsrc(tile_base, 0x7fffffffu);

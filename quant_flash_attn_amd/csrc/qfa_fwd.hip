@@ -1,7 +1,9 @@
 // Forward kernel: O = softmax(sm_scale * Q^ K^T) V with Q^, K^ given as per-token asymmetric
 // INT8 codes (scale, zero point, row sum per token).  gfx950, wave64.
 //
-// Work split.  One workgroup = 4 waves = 128 query rows of one (batch, head); each wave owns
+// Work split.  One workgroup = 4 waves = 128 query rows of one (batch, head) (8 waves per workgroup
+// halve the tile copies per query but measured 9 % slower: the barrier then waits for the slowest of
+// 8 waves); each wave owns
 // 32 queries.  K (3 buffers) and V (2 buffers) stream through LDS in tiles of 64 keys, copied by
 // direct global->LDS loads (no staging registers, no address or repacking work on the vector
 // pipe); K and the per-key constants are resident one tile ahead of V because the score product
@@ -47,8 +49,10 @@ namespace qfa {
 // correction, scaling and running maximum, with the exponentials and the P.V product compiled out
 // (it writes the scaled row maximum where the LSE would go and leaves O untouched).  It exists to
 // time the QK^T stage by itself against the INT8 MFMA peak.
-template <typename T, int D, bool CAUSAL, bool QK_ONLY = false>
-__global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
+template <typename T, int D, bool CAUSAL, bool QK_ONLY = false, int NW = FWD_WAVES>
+__global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
+  constexpr int NT = 64 * NW;        // threads per workgroup
+  constexpr int FWD_BM = 32 * NW;    // queries per workgroup
   typedef FwdSmem<D> SM;
   constexpr int KS = D / 32;   // int8 k-steps of 32
   constexpr int DB = D / 32;   // 32-row blocks of O^T
@@ -107,22 +111,12 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
   float c_sk;
   int c_rk, c_zk;
 
-  // Per-thread byte offsets of its 16-byte chunks inside a full tile (row * stride + swizzled chunk);
-  // the tile's first row goes into the wave-uniform base, so a full tile costs no address arithmetic
-  // on the vector pipe.  Ragged tiles (rows clamped to the last key) take the generic path.
-  constexpr int KCH = FWD_BN * (D / 16) / 256;        // K chunks per thread
-  constexpr int VCH = FWD_BN * (2 * D / 16) / 256;    // V chunks per thread
-  unsigned koff[KCH], voff[VCH];
-#pragma unroll
-  for (int i = 0; i < KCH; ++i) {
-    const int p = tid + 256 * i, row = p / KSW::CPR, pos = p % KSW::CPR;
-    koff[i] = (unsigned)row * (unsigned)a.skn + (unsigned)((pos ^ KSW::swz(row)) << 4);
-  }
-#pragma unroll
-  for (int i = 0; i < VCH; ++i) {
-    const int p = tid + 256 * i, row = p / VSW::CPR, pos = p % VSW::CPR;
-    voff[i] = (unsigned)row * (unsigned)(a.svn * sizeof(T)) + (unsigned)((pos ^ VSW::swz(row)) << 4);
-  }
+  // Full tiles: per-thread chunk offsets computed once (TileCopy); ragged tiles (rows clamped to the
+  // last key) take the generic path.
+  TileCopy<D, FWD_BN, NT, KSW> cp_k;
+  TileCopy<2 * D, FWD_BN, NT, VSW> cp_v;
+  cp_k.init((unsigned)a.skn, tid);
+  cp_v.init((unsigned)(a.svn * sizeof(T)), tid);
 
   // Full tiles are copied through buffer descriptors rebased to the tile's first row (scalar
   // arithmetic), so a copy costs one instruction per 16-byte chunk and thread; the per-key constant
@@ -141,15 +135,10 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
   auto load_k = [&](int t, int buf) {
     const int j0 = t * FWD_BN;
     unsigned char *dst = smem + SM::OFF_K + buf * SM::K_BYTES;
-    if (j0 + FWD_BN <= a.Nk) {
-      const rsrc_t rs = make_rsrc(reinterpret_cast<const unsigned char *>(kc_bh) + (int64_t)j0 * a.skn, 0x7fffffffu);
-#pragma unroll
-      for (int i = 0; i < KCH; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lptr_t)(dst + (wave_u * 64 + 256 * i) * 16), 16, (int)koff[i], 0, 0,
-                                                 0);
-    } else {
-      dma_rows<D, FWD_BN, 256, KSW>(reinterpret_cast<const unsigned char *>(kc_bh), a.skn, j0, a.Nk - 1, dst, tid);
-    }
+    if (j0 + FWD_BN <= a.Nk)
+      cp_k.issue(reinterpret_cast<const unsigned char *>(kc_bh) + (int64_t)j0 * a.skn, dst, wave_u, tid);
+    else
+      dma_rows<D, FWD_BN, NT, KSW>(reinterpret_cast<const unsigned char *>(kc_bh), a.skn, j0, a.Nk - 1, dst, tid);
     load_kc(t);
   };
   auto store_k = [&](int buf) {
@@ -166,15 +155,10 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
     const int j0 = t * FWD_BN;
     unsigned char *dst = smem + SM::OFF_V + (t & 1) * SM::V_BYTES;
     const int64_t vstride = a.svn * (int64_t)sizeof(T);
-    if (j0 + FWD_BN <= a.Nk) {
-      const rsrc_t rs = make_rsrc(reinterpret_cast<const unsigned char *>(v_bh) + (int64_t)j0 * vstride, 0x7fffffffu);
-#pragma unroll
-      for (int i = 0; i < VCH; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lptr_t)(dst + (wave_u * 64 + 256 * i) * 16), 16, (int)voff[i], 0, 0,
-                                                 0);
-    } else {
-      dma_rows<2 * D, FWD_BN, 256, VSW>(reinterpret_cast<const unsigned char *>(v_bh), vstride, j0, a.Nk - 1, dst, tid);
-    }
+    if (j0 + FWD_BN <= a.Nk)
+      cp_v.issue(reinterpret_cast<const unsigned char *>(v_bh) + (int64_t)j0 * vstride, dst, wave_u, tid);
+    else
+      dma_rows<2 * D, FWD_BN, NT, VSW>(reinterpret_cast<const unsigned char *>(v_bh), vstride, j0, a.Nk - 1, dst, tid);
   };
   // this lane's read offsets inside a tile (the swizzle terms only depend on the lane)
   const int k_swz = KSW::swz(lr);                                        // rows 32*nb + lr
@@ -333,7 +317,9 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
     // one body: V block (vbuf, nb); scores of the next block from kf; its constants in (cbuf, cnb);
     // then kf is refilled from K block (kbuf, knb).  `count_max`: whether the next block's maximum
     // may move the reference (false when that block belongs to a masked tile and is recomputed there).
-    auto body = [&](int vbuf, auto nb_tag, int cbuf, int cnb, int kbuf, int knb, bool count_max) {
+    // `copy(i)`, i = 0..2, is called between phases: the steady loop issues one chunk of the next
+    // tiles' copies there, so that the memory pipe sees single requests instead of a burst per tile
+    auto body = [&](int vbuf, auto nb_tag, int cbuf, int cnb, int kbuf, int knb, bool count_max, auto &&copy) {
       static_assert(DB == 4 || DB == 2, "fragment arrays are sized for head_dim 128 or 64");
       u32x2 vr0[2 * DB], vr1[2 * DB];
       u32x4 pf0, pf1;
@@ -348,6 +334,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
       for (int ks = 0; ks < KS; ++ks) s = mfma_i8(kf[ks], qf[ks], s);
       if (!QK_ONLY) exp_half(0, pf0);
       __builtin_amdgcn_sched_barrier(0);
+      copy(std::integral_constant<int, 0>{});
       if (!QK_ONLY) {
         v_frags(vbuf, NB, std::integral_constant<int, 1>{}, vr1);
         lds_wait_async<2 * DB>(vr0);   // the 2*DB requests just made may still be in flight
@@ -368,6 +355,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
       }
       __builtin_amdgcn_sched_barrier(0);
       if (!QK_ONLY) lds_wait_async<0>(vr1);   // everything requested so far was requested a phase ago
+      copy(std::integral_constant<int, 1>{});
       k_frags(kbuf, knb);
       __builtin_amdgcn_sched_barrier(0);
       f32x16 f;
@@ -385,6 +373,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
       __builtin_amdgcn_sched_barrier(0);
+      copy(std::integral_constant<int, 2>{});
       f = mfma_16b<T>(corr_k, corr_q, f);
       if (!QK_ONLY) {
 #pragma unroll
@@ -414,11 +403,35 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(FwdArgs a) {
       for (int v = 0; v < 16; ++v) u[v] = u0[v];
       k_frags(0, 1);
     }
+    auto no_copy = [](auto) {};
+    // steady state: K(t+2) and V(t+1) are full tiles; their chunks (K first, then V) go out one at a
+    // time between the phases of the two bodies
+    for (; t < t_hot && t + 2 < ntiles && (t + 3) * FWD_BN <= a.Nk; ++t) {
+      load_kc(t + 2);
+      const rsrc_t rs_k =
+          make_rsrc(reinterpret_cast<const unsigned char *>(kc_bh) + (int64_t)(t + 2) * FWD_BN * a.skn, 0x7fffffffu);
+      const rsrc_t rs_v = make_rsrc(
+          reinterpret_cast<const unsigned char *>(v_bh) + (int64_t)(t + 1) * FWD_BN * a.svn * (int64_t)sizeof(T), 0x7fffffffu);
+      unsigned char *kd = smem + SM::OFF_K + kb_free * SM::K_BYTES, *vd = smem + SM::OFF_V + ((t + 1) & 1) * SM::V_BYTES;
+      constexpr int KCH = decltype(cp_k)::N, VCH = decltype(cp_v)::N;
+      auto chunk = [&](int i) {   // i is a compile-time constant at every call site
+        if (i < KCH) cp_k.issue_one(rs_k, kd, wave_u, tid, i);
+        else if (i < KCH + VCH) cp_v.issue_one(rs_v, vd, wave_u, tid, i - KCH);
+      };
+      body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, true, [&](auto i) { chunk(decltype(i)::value); });
+      body(t & 1, std::integral_constant<int, 1>{}, kb_nxt, 0, kb_nxt, 1, t + 1 < t_hot,
+           [&](auto i) { chunk(3 + decltype(i)::value); });
+      static_assert(KCH + VCH <= 6, "six copy slots per tile");
+      store_k(kb_free);
+      const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
+      dma_wait();
+      __syncthreads();
+    }
     for (; t < t_hot; ++t) {
       if (t + 2 < ntiles) load_k(t + 2, kb_free);
       if (t + 1 < ntiles) load_v(t + 1);
-      body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, true);
-      body(t & 1, std::integral_constant<int, 1>{}, kb_nxt, 0, kb_nxt, 1, t + 1 < t_hot);
+      body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, true, no_copy);
+      body(t & 1, std::integral_constant<int, 1>{}, kb_nxt, 0, kb_nxt, 1, t + 1 < t_hot, no_copy);
       if (t + 2 < ntiles) store_k(kb_free);
       const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
       dma_wait();
@@ -477,12 +490,13 @@ template <typename T, int D> static int launch_fwd_td(const AttnArgs &x, hipStre
   a.sqb = x.sqb; a.sqh = x.sqh; a.sqn = x.sqn; a.skb = x.skb; a.skh = x.skh; a.skn = x.skn;
   a.svb = x.svb; a.svh = x.svh; a.svn = x.svn; a.sob = x.sob; a.soh = x.soh; a.son = x.son;
   a.sm_scale_log2 = x.sm_scale * kLog2e;
+  constexpr int FWD_BM = 32 * FWD_WAVES;
   a.mblocks = (int)((x.Nq + FWD_BM - 1) / FWD_BM);
   const int64_t total = (int64_t)a.mblocks * x.B * x.H;
   if (total > 0x3fffffffLL) return set_error(QFA_EUNSUPPORTED, "attn_fwd: too many query blocks for one launch");
   a.total_blocks = (int)total;
   a.blocks_per_xcd = (a.total_blocks + 7) / 8;
-  const dim3 grid((unsigned)(a.blocks_per_xcd * 8)), block(256);
+  const dim3 grid((unsigned)(a.blocks_per_xcd * 8)), block(64 * FWD_WAVES);
   if (qk_only) {
     if (x.causal) fwd_kernel<T, D, true, true><<<grid, block, 0, st>>>(a);
     else fwd_kernel<T, D, false, true><<<grid, block, 0, st>>>(a);

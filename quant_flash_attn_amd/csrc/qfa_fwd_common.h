@@ -13,12 +13,15 @@ struct FwdArgs {
   int Nq, Nk;
   int64_t sqb, sqh, sqn, skb, skh, skn, svb, svh, svn, sob, soh, son;
   float sm_scale_log2;   // sm_scale * log2(e)
-  int mblocks;           // ceil(Nq / 128)
+  int mblocks;           // query blocks of one workgroup each per (batch, head)
   int total_blocks;      // mblocks * B * H
   int blocks_per_xcd;    // ceil(total_blocks / 8)
 };
 
-constexpr int FWD_BM = 128;
+#ifndef QFA_FWD_WAVES
+#define QFA_FWD_WAVES 4
+#endif
+constexpr int FWD_WAVES = QFA_FWD_WAVES;   // waves (32 queries each) per workgroup
 constexpr int FWD_BN = 64;
 constexpr float FWD_RESCALE_THRESHOLD = 8.0f;   // log2 units the running max may lag behind
 
