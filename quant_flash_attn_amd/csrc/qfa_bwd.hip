@@ -317,9 +317,10 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(BwdArgs a) {
   cp_v.init((unsigned)a.svn * 2u, tid);
   cp_t.init(BWD_TILE * 2, tid);
   cp_c.init(0, tid);
-  auto load_tile = [&](int t) {
+  // the copy of a tile goes out in two halves (one before each 32-key block of the tile in work), so
+  // that the memory pipe is not handed all of it in one burst
+  auto load_tile_a = [&](int t) {
     unsigned char *base = smem + (t & 1) * BUF;
-    const unsigned char *blob = wsk_bh + (int64_t)t * WS::K_BLOB;
     if ((t + 1) * BWD_TILE <= a.Nk) {
       cp_k.issue(kc_bh + (int64_t)t * BWD_TILE * a.skn, base, wave_u, tid);
       cp_v.issue(v_bh + (int64_t)t * BWD_TILE * a.svn * 2, base + OFF_V, wave_u, tid);
@@ -327,8 +328,16 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(BwdArgs a) {
       dma_rows<D, BWD_TILE, DQ_THREADS>(kc_bh, a.skn, t * BWD_TILE, a.Nk - 1, base, tid);
       dma_rows<2 * D, BWD_TILE, DQ_THREADS>(v_bh, a.svn * 2, t * BWD_TILE, a.Nk - 1, base + OFF_V, tid);
     }
+  };
+  auto load_tile_b = [&](int t) {
+    unsigned char *base = smem + (t & 1) * BUF;
+    const unsigned char *blob = wsk_bh + (int64_t)t * WS::K_BLOB;
     cp_t.issue(blob, base + OFF_T, wave_u, tid);
     cp_c.issue(blob + WS::T_BYTES, base + OFF_C, wave_u, tid);
+  };
+  auto load_tile = [&](int t) {
+    load_tile_a(t);
+    load_tile_b(t);
   };
 
   f32x16 dqacc[DB];
@@ -396,10 +405,13 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(BwdArgs a) {
   dma_wait();
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
-    if (t + 1 < ntiles) load_tile(t + 1);
     const int j0 = t * BWD_TILE;
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
+      if (t + 1 < ntiles) {
+        if (nb == 0) load_tile_a(t + 1);
+        else load_tile_b(t + 1);
+      }
       const int jb = j0 + 32 * nb;
       if ((jb >= a.Nk) || (CAUSAL && jb > q_last)) continue;               // wave-uniform
       if ((CAUSAL && jb + 31 > q_first) || (jb + 32 > a.Nk)) block(t, nb, std::true_type{});
@@ -501,19 +513,28 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
   cp_g.init((unsigned)a.sdon * 2u, tid);
   cp_t.init(BWD_TILE * 2, tid);
   cp_c.init(0, tid);
-  auto load_tile = [&](int t) {
+  // the copy of a tile goes out in two halves (parts 0-1, 2-3), one before each 32-query block of the
+  // tile in work, so that the memory pipe is not handed all of it in one burst (four quarters, one
+  // per phase, measured slower)
+  auto load_part = [&](int t, int part) {
     unsigned char *base = smem + (t & 1) * BUF;
     const unsigned char *blob = wsq_bh + (int64_t)t * WS::Q_BLOB;
-    if ((t + 1) * BWD_TILE <= a.Nq) {
-      cp_q.issue(qc_bh + (int64_t)t * BWD_TILE * a.sqn, base, wave_u, tid);
-      cp_g.issue(do_bh + (int64_t)t * BWD_TILE * a.sdon * 2, base + OFF_DO, wave_u, tid);
+    const bool full = (t + 1) * BWD_TILE <= a.Nq;
+    if (part == 0) {
+      if (full) cp_q.issue(qc_bh + (int64_t)t * BWD_TILE * a.sqn, base, wave_u, tid);
+      else dma_rows<D, BWD_TILE, DKV_THREADS>(qc_bh, a.sqn, t * BWD_TILE, a.Nq - 1, base, tid);
+      cp_c.issue(blob + 2 * WS::T_BYTES, base + OFF_C, wave_u, tid);
+    } else if (part == 1) {
+      if (full) cp_g.issue(do_bh + (int64_t)t * BWD_TILE * a.sdon * 2, base + OFF_DO, wave_u, tid);
+      else dma_rows<2 * D, BWD_TILE, DKV_THREADS>(do_bh, a.sdon * 2, t * BWD_TILE, a.Nq - 1, base + OFF_DO, tid);
+    } else if (part == 2) {
+      cp_t.issue(blob, base + OFF_DOT, wave_u, tid);
     } else {
-      dma_rows<D, BWD_TILE, DKV_THREADS>(qc_bh, a.sqn, t * BWD_TILE, a.Nq - 1, base, tid);
-      dma_rows<2 * D, BWD_TILE, DKV_THREADS>(do_bh, a.sdon * 2, t * BWD_TILE, a.Nq - 1, base + OFF_DO, tid);
+      cp_t.issue(blob + WS::T_BYTES, base + OFF_QT, wave_u, tid);
     }
-    cp_t.issue(blob, base + OFF_DOT, wave_u, tid);
-    cp_t.issue(blob + WS::T_BYTES, base + OFF_QT, wave_u, tid);
-    cp_c.issue(blob + 2 * WS::T_BYTES, base + OFF_C, wave_u, tid);
+  };
+  auto load_tile = [&](int t) {
+    for (int part = 0; part < 4; ++part) load_part(t, part);
   };
 
   f32x16 oacc[DB];   // dV^T (P role) or dK^T (dS role) for this lane's key
@@ -649,10 +670,13 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
   };
   if (p_role) {
     for (int t = it0; t < ntiles; ++t) {
-      if (t + 1 < ntiles) load_tile(t + 1);
       const unsigned char *base = smem + (t & 1) * BUF;
 #pragma unroll
       for (int mbk = 0; mbk < 2; ++mbk) {
+        if (t + 1 < ntiles) {
+          load_part(t + 1, 2 * mbk);
+          load_part(t + 1, 2 * mbk + 1);
+        }
         bool on, masked;
         block_flags(t, mbk, on, masked);
         u32x4 pf[2], tf[2 * DB];
@@ -673,10 +697,13 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
     }
   } else {
     for (int t = it0; t < ntiles; ++t) {
-      if (t + 1 < ntiles) load_tile(t + 1);
       const unsigned char *base = smem + (t & 1) * BUF;
 #pragma unroll
       for (int mbk = 0; mbk < 2; ++mbk) {
+        if (t + 1 < ntiles) {
+          load_part(t + 1, 2 * mbk);
+          load_part(t + 1, 2 * mbk + 1);
+        }
         bool on, masked;
         block_flags(t, mbk, on, masked);
         u32x4 dsf[2], tf[2 * DB];
