@@ -83,7 +83,7 @@ int qfa_dequant_per_token(const int8_t *codes, const void *scale, int scale_dtyp
  *   qc,kc  int8 [B,H,Nq|Nk,D];  sq,sk float, zq,zk int8, rq,rk int32: dense [B*H*Nq|Nk]
  *   v, o   [B,H,Nk|Nq,D] of io_dtype (QFA_BF16 or QFA_F16);  lse float [B*H*Nq]
  *   D in {64, 128}.  causal != 0 requires Nq == Nk.  All tensors 16-byte aligned, strides
- *   multiples of 16 bytes.
+ *   multiples of 16 bytes, token strides below 2^23 elements (QFA_EUNSUPPORTED otherwise).
  */
 int qfa_attn_fwd(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,
                  const float *sk, const int8_t *zk, const int32_t *rk, const void *v, void *o, float *lse,

@@ -52,6 +52,12 @@ def test_argument_errors_need_no_gpu(qfa):
     assert fwd(sm=0.0) == -1 and b"sm_scale" in L.qfa_last_error()
     assert fwd(D=96) == -2 and b"head_dim" in L.qfa_last_error()
     assert fwd(io=0) == -1 and b"io_dtype" in L.qfa_last_error()
+    # token strides of 2^23 elements or more: tile-relative offsets would not fit 31 bits
+    big = (1 << 23)
+    sb = (2 * 128 * big, 128 * big, big)
+    s0 = (128 * 64 * 2, 128 * 64, 64)
+    rc = L.qfa_attn_fwd(*([ok_ptr] * 11), 2, 1, 2, 128, 128, 64, *s0, *sb, *s0, *s0, 0.125, 0, None)
+    assert rc == -2 and b"token strides" in L.qfa_last_error()
     rc = L.qfa_bwd_delta(None, ok_ptr, ok_ptr, 2, 1, 1, 8, 64, 512, 512, 64, 512, 512, 64, None)
     assert rc == -1
 
