@@ -458,8 +458,8 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
   constexpr int Q_BYTES = BWD_TILE * D, G_BYTES = BWD_TILE * 2 * D, T_BYTES = WS::T_BYTES;
   constexpr int OFF_DO = Q_BYTES, OFF_DOT = OFF_DO + G_BYTES, OFF_QT = OFF_DOT + T_BYTES, OFF_C = OFF_QT + T_BYTES,
                 BUF = OFF_C + WS::CQ_BYTES;
-  constexpr int OFF_X = 2 * BUF;             // P exchange: 4 pairs x 64 lanes x 16 floats
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF + 4 * 4096];
+  constexpr int OFF_X = 2 * BUF;             // P exchange: 2 slots x 4 pairs x 64 lanes x 16 floats
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF + 2 * 4 * 4096];
 
   const int L = blockIdx.x;
   const int vid = (L % 8) * a.blocks_per_xcd + (L / 8);
@@ -543,7 +543,9 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) oacc[db][v] = 0.f;
 
-  f32x4 *xch = reinterpret_cast<f32x4 *>(smem + OFF_X + pair * 4096);   // [4][64 lanes] of 4 floats
+  // [slot][4][64 lanes] of 4 floats; the slot is the block's parity, so that one barrier per block is
+  // enough: P(b) is written before barrier b and read before barrier b+1, P(b+2) is written after it
+  f32x4 *xch0 = reinterpret_cast<f32x4 *>(smem + OFF_X + pair * 4096);
 
   // LDS operands are fetched in groups well ahead of the MFMAs that consume them (a 16-byte LDS read
   // takes far longer than an MFMA issue slot, and the compiler keeps loads next to their use), the
@@ -591,7 +593,7 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
         pp[4 * aa + bb] = p;
         p4[bb] = p;
       }
-      xch[aa * 64 + lane] = p4;
+      xch0[mbk * 1024 + aa * 64 + lane] = p4;
     }
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh)
@@ -636,10 +638,10 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
       for (int db = 0; db < DB; ++db) oacc[db] = mfma_16b<T>(tf[hh * DB + db], bf[hh], oacc[db]);
   };
   // ---- dS role, second half prologue: dS' = P (from partner) * (dP - delta) * a, packed
-  auto ds_second = [&](const f32x16 &dp, const f32x4 (&a4)[4], const f32x4 (&dl4)[4], u32x4 (&dsf)[2]) {
+  auto ds_second = [&](int mbk, const f32x16 &dp, const f32x4 (&a4)[4], const f32x4 (&dl4)[4], u32x4 (&dsf)[2]) {
     f32x4 p4[4];
 #pragma unroll
-    for (int aa = 0; aa < 4; ++aa) p4[aa] = xch[aa * 64 + lane];
+    for (int aa = 0; aa < 4; ++aa) p4[aa] = xch0[mbk * 1024 + aa * 64 + lane];
     float ds[16];
 #pragma unroll
     for (int aa = 0; aa < 4; ++aa)
@@ -651,48 +653,41 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
       for (int e = 0; e < 4; ++e) dsf[hh][e] = pack2<T>(ds[8 * hh + 2 * e], ds[8 * hh + 2 * e + 1]);
   };
 
-#ifdef QFA_TIMING
-  long long tacc[5] = {0, 0, 0, 0, 0};
-  long long tprev = clock64();
-#define QFA_TICK(i) { const long long tn = clock64(); tacc[i] += tn - tprev; tprev = tn; }
-#else
-#define QFA_TICK(i)
-#endif
   if (it0 < ntiles) load_tile(it0);
   dma_wait();
   __syncthreads();
-  QFA_TICK(0)
-  // The two roles run separate loops with the same barrier sequence (2 per 32-query block).
+  // The two roles run separate loops with the same barrier sequence (one per 32-query block).
   auto block_flags = [&](int t, int mbk, bool &on, bool &masked) {
     const int ib = t * BWD_TILE + 32 * mbk;
     on = (ib < a.Nq) && (!CAUSAL || ib + 31 >= k_first);                               // wave-uniform
     masked = (CAUSAL && ib < k_last) || (ib + 32 > a.Nq) || (k_last >= a.Nk);
   };
+  // Block (t, mbk): first phase | barrier | second phase.  The next tile's copy goes out in two halves
+  // around the barrier of the tile's first block and must have landed before the barrier of its
+  // second block (its buffer was last read before the previous tile's last barrier).
   if (p_role) {
     for (int t = it0; t < ntiles; ++t) {
       const unsigned char *base = smem + (t & 1) * BUF;
 #pragma unroll
       for (int mbk = 0; mbk < 2; ++mbk) {
-        if (t + 1 < ntiles) {
-          load_part(t + 1, 2 * mbk);
-          load_part(t + 1, 2 * mbk + 1);
+        if (mbk == 0 && t + 1 < ntiles) {
+          load_part(t + 1, 0);
+          load_part(t + 1, 1);
         }
         bool on, masked;
         block_flags(t, mbk, on, masked);
         u32x4 pf[2], tf[2 * DB];
-        QFA_TICK(0)
         if (on) {
           if (masked) p_first(base, t * BWD_TILE, mbk, pf, tf, std::true_type{});
           else p_first(base, t * BWD_TILE, mbk, pf, tf, std::false_type{});
         }
-        QFA_TICK(1)
-        lds_barrier();   // P of this block is in LDS (the next tile's direct loads stay in flight)
-        QFA_TICK(2)
-        if (on) accumulate(tf, pf);
-        QFA_TICK(3)
         if (mbk == 1) dma_wait();
-        lds_barrier();   // P consumed; after the second block the next tile has landed
-        QFA_TICK(4)
+        lds_barrier();   // P of this block is in LDS
+        if (mbk == 0 && t + 1 < ntiles) {
+          load_part(t + 1, 2);
+          load_part(t + 1, 3);
+        }
+        if (on) accumulate(tf, pf);
       }
     }
   } else {
@@ -700,38 +695,29 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
       const unsigned char *base = smem + (t & 1) * BUF;
 #pragma unroll
       for (int mbk = 0; mbk < 2; ++mbk) {
-        if (t + 1 < ntiles) {
-          load_part(t + 1, 2 * mbk);
-          load_part(t + 1, 2 * mbk + 1);
+        if (mbk == 0 && t + 1 < ntiles) {
+          load_part(t + 1, 0);
+          load_part(t + 1, 1);
         }
         bool on, masked;
         block_flags(t, mbk, on, masked);
         u32x4 dsf[2], tf[2 * DB];
         f32x16 dp;
         f32x4 a4[4], dl4[4];
-        QFA_TICK(0)
         if (on) ds_first(base, mbk, dp, tf, a4, dl4);
-        QFA_TICK(1)
-        lds_barrier();
-        QFA_TICK(2)
-        if (on) {
-          ds_second(dp, a4, dl4, dsf);
-          accumulate(tf, dsf);
-        }
-        QFA_TICK(3)
         if (mbk == 1) dma_wait();
         lds_barrier();
-        QFA_TICK(4)
+        if (mbk == 0 && t + 1 < ntiles) {
+          load_part(t + 1, 2);
+          load_part(t + 1, 3);
+        }
+        if (on) {
+          ds_second(mbk, dp, a4, dl4, dsf);
+          accumulate(tf, dsf);
+        }
       }
     }
   }
-#ifdef QFA_TIMING
-  if (lane == 0 && bh == 0) {
-    long long *out = reinterpret_cast<long long *>(a.dq) + (nbk * 8 + wave) * 8;
-    for (int i = 0; i < 5; ++i) out[i] = tacc[i];
-    out[5] = ntiles - it0;
-  }
-#endif
 
   if (kj < a.Nk) {
     T *row = (p_role ? dv_bh + (int64_t)kj * a.sdvn : dk_bh + (int64_t)kj * a.sdkn);
@@ -793,10 +779,8 @@ template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStre
     a.total_blocks = (int)total;
     a.blocks_per_xcd = (a.total_blocks + 7) / 8;
     const dim3 grid((unsigned)(a.blocks_per_xcd * 8));
-#ifndef QFA_TIMING
     if (x.causal) bwd_dq_kernel<T, D, true><<<grid, dim3(DQ_THREADS), 0, st>>>(a);
     else bwd_dq_kernel<T, D, false><<<grid, dim3(DQ_THREADS), 0, st>>>(a);
-#endif
     if (int e = check_launch("qfa_attn_bwd (dq)")) return e;
   }
   return 0;
