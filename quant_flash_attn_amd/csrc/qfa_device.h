@@ -200,20 +200,14 @@ __device__ __forceinline__ void dma_flat(const unsigned char *g, unsigned char *
 }
 // all direct loads of this wave have landed (vmcnt(0)); follow with a barrier before other waves read
 __device__ __forceinline__ void dma_wait() { __builtin_amdgcn_s_waitcnt(0x0f70); }
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
-// global access, including direct-to-LDS loads issued for a LATER tile, which would serialise the
-// prefetch; this one leaves them in flight (pair it with dma_wait() where a tile must have landed).
 // ds_read_b64_tr_b16: inside each group of 16 lanes, lane i receives element i%4 of the four 8-byte
 // rows addressed by lanes (i%16)/4, +4, +8, +12 of its group -- a 16-bit transpose on the way out of LDS.
-__device__ __forceinline__ u32x2 lds_read_tr16(const unsigned char *p) {
-  typedef short s16x4 __attribute__((ext_vector_type(4)));
-  return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p));
-}
-// The same read issued behind the compiler's back, with an explicit wait.  The compiler makes every
-// ds_read_b64_tr_b16 it knows of wait for ALL outstanding direct-to-LDS loads (it cannot tell which
-// buffer they fill), which would expose the latency of the next tile's copy once per tile.  The asm
-// form is invisible to that bookkeeping, so the result must not be used before one of the waits
-// below, which take the loaded registers as operands to keep their consumers behind them.
+// It is issued behind the compiler's back, with an explicit wait: the compiler makes every such read
+// it knows of (__builtin_amdgcn_ds_read_tr16_b64) wait for ALL outstanding direct-to-LDS loads (it
+// cannot tell which buffer they fill), which would expose the latency of the next tile's copy once
+// per tile.  The asm form is invisible to that bookkeeping, so the result must not be used before
+// one of the waits below, which take the loaded registers as operands to keep their consumers
+// behind them.
 // LDS operations return in order: lgkmcnt(N) guarantees everything but the last N issued is there.
 __device__ __forceinline__ unsigned lds_addr(const void *p) { return (unsigned)(size_t)(lptr_t)p; }
 template <int OFF> __device__ __forceinline__ u32x2 lds_read_tr16_async(unsigned addr) {
@@ -230,6 +224,9 @@ template <int N> __device__ __forceinline__ void lds_wait_async(u32x2 (&r)[8]) {
 template <int N> __device__ __forceinline__ void lds_wait_async(u32x2 (&r)[4]) {
   asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]) : "n"(N) : "memory");
 }
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
+// global access, including direct-to-LDS loads issued for a LATER tile, which would serialise the
+// prefetch; this one leaves them in flight (pair it with dma_wait() where a tile must have landed).
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 }  // namespace qfa

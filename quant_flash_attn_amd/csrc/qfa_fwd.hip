@@ -239,9 +239,18 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
       l_run = fmaxf(l_run, s);
       return;
     }
-    const unsigned char *vt_ = smem + SM::OFF_V + vbuf * SM::V_BYTES;
+    // keys 32nb + 16hh + 4g + {0..3} and those + 8: the order in which pf holds the probabilities.
+    // The reads are issued behind the compiler's back (see lds_read_tr16_async) and waited for below.
+    const unsigned vbase = lds_addr(smem + SM::OFF_V) + vbuf * SM::V_BYTES + (32 * nb + 4 * g) * SM::VSTR;
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh) {
+      u32x2 vr[2 * DB];
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const unsigned ad = vbase + hh * (16 * SM::VSTR) + (v_off ^ (64 * db));
+        vr[2 * db] = lds_read_tr16_async<0>(ad);
+        vr[2 * db + 1] = lds_read_tr16_async<8 * SM::VSTR>(ad);
+      }
       u32x4 pf;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -250,14 +259,10 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
         pf[e] = pack2<T>(p0, p1);
         l_run = dot2_ones<T>(pf[e], l_run);   // sum of the rounded pair, fp32 accumulate
       }
+      lds_wait_async<0>(vr);
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        // keys 32nb + 16hh + 4g + {0..3} and those + 8: the order in which pf holds the probabilities
-        const unsigned char *vp = vt_ + (32 * nb + 16 * hh + 4 * g) * SM::VSTR + (v_off ^ (64 * db));
-        const u32x2 v0 = lds_read_tr16(vp), v1 = lds_read_tr16(vp + 8 * SM::VSTR);
-        const u32x4 vf = {v0[0], v0[1], v1[0], v1[1]};
-        oacc[db] = mfma_16b<T>(vf, pf, oacc[db]);
-      }
+      for (int db = 0; db < DB; ++db)
+        oacc[db] = mfma_16b<T>(u32x4{vr[2 * db][0], vr[2 * db][1], vr[2 * db + 1][0], vr[2 * db + 1][1]}, pf, oacc[db]);
     }
   };
 

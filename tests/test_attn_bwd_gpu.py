@@ -120,7 +120,8 @@ def test_autograd_entry_points(qfa):
     assert_close("dV", vg.grad.cpu(), rv, scaled=True)
 
 
-@pytest.mark.parametrize("Z,H,Nq,Nkv,D", [(2, 4, 18, 512, 64), (2, 8, 32, 1024, 128), (1, 2, 17, 1023, 128), (3, 5, 97, 689, 128)])
+@pytest.mark.parametrize("Z,H,Nq,Nkv,D", [(2, 4, 18, 512, 64), (2, 8, 32, 1024, 128), (4, 16, 16, 2048, 64), (1, 2, 17, 1023, 128),
+                                          (3, 5, 97, 689, 128)])
 def test_reference_entry_point_shared_kv(qfa, Z, H, Nq, Nkv, D):
     """The reference's own test (test_accuracy.py:47-133): fp16 q, kv ~ N(0,1), seed 20, quantize kv
     externally, forward + backward, against un-quantized fp16-input attention at its tolerances
