@@ -184,6 +184,8 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) oacc[db][v] = 0.f;
   float m_ref = -INFINITY;   // reference maximum of u = score / a_i used in the exponent
+  float m_bound = -INFINITY;                        // m_ref + threshold / a_i
+  const float thr_i = FWD_RESCALE_THRESHOLD / a_i;
   float nm = INFINITY;       // -a_i * m_ref
   float l_run = 0.f;         // this lane's share of the row sum
 
@@ -217,11 +219,14 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
     return max_across_halves(mt);
   };
   // move the reference maximum only when some row of the wave outgrew it by > 2^threshold
+  // (the test is one compare against m_ref + threshold / a_i, kept in m_bound: it sits at the end
+  // of a dependent chain that nothing else in the wave can overlap)
   auto rescale_if_needed = [&](float mt) {
-    if (__builtin_amdgcn_ballot_w64(a_i * (mt - m_ref) > FWD_RESCALE_THRESHOLD) != 0) {
+    if (__builtin_amdgcn_ballot_w64(mt > m_bound) != 0) {
       const float m_new = fmaxf(m_ref, mt);
       const float alpha = __builtin_amdgcn_exp2f(a_i * (m_ref - m_new));
       m_ref = m_new;
+      m_bound = m_new + thr_i;
       nm = -a_i * m_new;
       l_run *= alpha;
 #pragma unroll
@@ -387,15 +392,16 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
         for (int e = 0; e < 4; ++e) l_run = dot2_ones<T>(pf1[e], l_run);
       }
       __builtin_amdgcn_sched_barrier(0);
-      float mt = -INFINITY;
+      float mt0 = -INFINITY, mt1 = -INFINITY;   // two chains: half the dependent latency
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa)
 #pragma unroll
         for (int bb = 0; bb < 4; ++bb) {
           u[4 * aa + bb] = f[4 * aa + bb] * sk4[aa][bb];
-          mt = fmaxf(mt, u[4 * aa + bb]);
+          if (aa & 1) mt1 = fmaxf(mt1, u[4 * aa + bb]);
+          else mt0 = fmaxf(mt0, u[4 * aa + bb]);
         }
-      mt = max_across_halves(mt);
+      float mt = max_across_halves(fmaxf(mt0, mt1));
       rescale_if_needed(count_max ? mt : -INFINITY);
     };
 
