@@ -41,4 +41,15 @@ int launch_delta(const void *o, const void *dout, float *delta, int io_dtype, in
 int launch_bwd(const AttnArgs &a, hipStream_t st);
 int64_t bwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D);
 
+// Shared-KV attention (K = V = one quantized tensor, Q in 16-bit float), after validation.
+struct SkvAttnArgs {
+  const void *q; const int8_t *codes; const void *scale; const int8_t *zp;
+  void *o; float *lse;
+  int64_t B, H, Nq, Nk;
+  int64_t sqb, sqh, sqn, scb, sch, scn, sob, soh, son;
+  float sm_scale;
+  int D, io_dtype, scale_dtype;
+};
+int launch_skv_fwd(const SkvAttnArgs &a, hipStream_t st);
+
 }  // namespace qfa

@@ -1,0 +1,386 @@
+// Shared-KV attention for short query blocks: the reference's own operator and benchmark shape
+// (quant_flash_attn.py:22-83; compute_flops.py:96: Z=512, H=16, 16 queries against 3000 keys).
+//     O = softmax(sm_scale * Q K^^T) K^,    K^ = V^ = scale * (codes - zero_point)  per token,
+// with Q left in 16-bit floating point exactly as the reference does (:50-52).  The operator is
+// bound by reading the INT8 codes once: per (batch, head) there are only a few queries, so the
+// kernel streams the codes -- and nothing else -- through LDS and keeps the matrix pipe fed from them.
+//
+// Work split.  One workgroup = 4 waves = one block of 32 queries of one (batch, head); the 32-key
+// tiles of the sequence are dealt round-robin to the waves, every wave runs its own online softmax
+// over its tiles from a private ring of LDS buffers filled by direct global->LDS loads (no
+// workgroup barrier in the loop), and the four partial results are merged at the end.
+//
+// Codes as MFMA operands.  A code byte c (two's complement) with its top bit flipped is the
+// unsigned byte c + 128; OR-ed under the constant 0x6400 it is the binary16 number 1152 + c
+// exactly, so one XOR per dword and one byte permute per pair of elements turn codes into a
+// 16-bit MFMA operand.  The offset is taken out again exactly:
+//     sum_d (1152 + c_jd) q_d  - (1152 + zp_j) * sum_d q_d        = sum_d (c_jd - zp_j) q_d
+//     sum_j (1152 + c_jd) p'_j - sum_j (1152 + zp_j) p'_j         = sum_j (c_jd - zp_j) p'_j
+// The first subtraction is a rank-1 update done by one more MFMA (sum_d q_d split into three
+// binary16 terms, products exact in fp32); the second is a per-query scalar accumulated with
+// v_dot2 over the same rounded p' = p * scale_j that the MFMA consumed, so the offsets cancel
+// exactly and only the usual rounding of P remains.
+//
+// V^T fragments come out of the row-major code tile through ds_read_b64_tr_b8: inside a group of 16
+// lanes, lane i receives byte i%8 of the 8-byte rows addressed by lanes (i%16)/8 + {0,2,..,14}.
+#include <type_traits>
+
+#include "qfa_device.h"
+#include "qfa_host.h"
+
+namespace qfa {
+
+struct SkvArgs {
+  const void *q; const int8_t *codes; const void *scale; const int8_t *zp;
+  void *o; float *lse;
+  int64_t H;
+  int Nq, Nk;
+  int64_t sqb, sqh, sqn, scb, sch, scn, sob, soh, son;
+  float sm_scale_log2;
+  int qblocks;   // ceil(Nq / 32)
+};
+
+constexpr int SKV_TILE = 32;     // keys per tile
+constexpr int SKV_NBUF = 4;      // ring depth per wave
+constexpr float SKV_RESCALE_THRESHOLD = 4.0f;   // p <= 2^4: p * scale stays inside binary16 for any fp16 K
+
+__device__ __forceinline__ f32x16 mfma_h(u32x4 a, u32x4 b, f32x16 c) { return mfma_16b<_Float16>(a, b, c); }
+// two unsigned bytes (positions A and A+1 of w) -> packed binary16 pair (1024 + byte)
+template <int A> __device__ __forceinline__ unsigned magic_pair(unsigned w) {
+  constexpr unsigned sel = 0x04000400u | (unsigned)A | ((unsigned)(A + 1) << 16);
+  return __builtin_amdgcn_perm(0x64646464u, w, sel);
+}
+// 8 code bytes (two dwords) -> 8 binary16 values 1152 + code
+__device__ __forceinline__ u32x4 expand_codes(unsigned w0, unsigned w1) {
+  w0 ^= 0x80808080u;
+  w1 ^= 0x80808080u;
+  return u32x4{magic_pair<0>(w0), magic_pair<2>(w0), magic_pair<0>(w1), magic_pair<2>(w1)};
+}
+__device__ __forceinline__ unsigned pack_h2(float a, float b) { return pack2<_Float16>(a, b); }
+// binary16 pair (1152 + za, 1152 + zb) from two zero points held in the low bytes of za and zb
+__device__ __forceinline__ unsigned magic_zp_pair(unsigned za, unsigned zb) {
+  return __builtin_amdgcn_perm(za, zb, 0x0c000c04u) ^ 0x64806480u;
+}
+// ds_read_b64_tr_b8, issued like lds_read_tr16_async: invisible to the compiler's wait bookkeeping
+// (which would make it wait for every direct-to-LDS load in flight), to be followed by lds_wait_async.
+__device__ __forceinline__ u32x2 lds_read_tr8_async(unsigned addr) {
+  u32x2 r;
+  asm volatile("ds_read_b64_tr_b8 %0, %1" : "=v"(r) : "v"(addr) : "memory");
+  return r;
+}
+
+template <int D> struct SkvSmem {
+  static constexpr int K_BYTES = SKV_TILE * D;             // codes of a tile, rows dense, chunks swizzled (Swz<D>)
+  static constexpr int SLOT = K_BYTES + 2 * SKV_TILE * 4;  // + one dword per key for the scale, one for the zero point
+  static constexpr int WAVE = SKV_NBUF * SLOT;
+  static constexpr int MG = 32 * D + 64;                   // floats of one partial result: O^T [D][32], m[32], l[32]
+  static constexpr int MERGE = 3 * MG * 4;
+  static constexpr int TOTAL = 4 * WAVE > MERGE ? 4 * WAVE : MERGE;
+};
+
+// T: element type of Q and O.  S: element type of the scale vector (float, or T).
+template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) void skv_fwd_kernel(SkvArgs a) {
+  typedef SkvSmem<D> SM;
+  typedef Swz<D> KSW;
+  typedef TileCopy<D, SKV_TILE, 64, KSW> Copy;
+  constexpr int KD = D / 16;    // 16-wide k-steps of the score product
+  constexpr int DB = D / 32;    // 32-row blocks of O^T
+  constexpr int OPS = Copy::N + 2;   // vector-memory instructions per tile
+  __shared__ __attribute__((aligned(16))) unsigned char smem[SM::TOTAL];
+
+  const int bh = blockIdx.x / a.qblocks, qb = blockIdx.x % a.qblocks;
+  const int64_t b = bh / a.H, h = bh % a.H;
+  const int tid = threadIdx.x, lane = tid % 64, lr = lane % 32, g = lane / 32;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  unsigned char *ring = smem + wave * SM::WAVE;
+
+  const unsigned char *codes_bh = reinterpret_cast<const unsigned char *>(a.codes + b * a.scb + h * a.sch);
+  const int64_t tk0 = (int64_t)bh * a.Nk, tq0 = (int64_t)bh * a.Nq;
+  const int ntiles = (a.Nk + SKV_TILE - 1) / SKV_TILE;
+  const int my_tiles = ntiles > wave ? (ntiles - wave + 3) / 4 : 0;    // tiles wave, wave+4, ...
+
+  // ---- this lane's query as binary16 B operand of the score product, and sum_d q_d
+  const int qi = qb * 32 + lr;
+  const int qi_c = qi < a.Nq ? qi : a.Nq - 1;
+  const T *qrow = reinterpret_cast<const T *>(a.q) + b * a.sqb + h * a.sqh + (int64_t)qi_c * a.sqn;
+  u32x4 qf[KD];
+  float rs = 0.f;
+#pragma unroll
+  for (int m = 0; m < KD; ++m) {
+    // k-step m = 2j + hf covers d = 32j + 16g + 8hf + {0..7}: the two halves of one 16-byte code chunk
+    const int d0 = 32 * (m / 2) + 16 * g + 8 * (m % 2);
+    const u32x4 raw = *reinterpret_cast<const u32x4 *>(qrow + d0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      // bf16 input enters through its binary16 rounding
+      qf[m][e] = std::is_same<T, _Float16>::value ? raw[e] : pack_h2(lo_to_f32<T>(raw[e]), hi_to_f32<T>(raw[e]));
+      rs += lo_to_f32<_Float16>(qf[m][e]) + hi_to_f32<_Float16>(qf[m][e]);
+    }
+  }
+  rs += swap32_f(rs);
+  // -sum_d q_d as three binary16 terms, k-group 0 of the correction MFMA's B operand
+  u32x4 corr_q = {0u, 0u, 0u, 0u};
+  {
+    const _Float16 h0 = (_Float16)rs;
+    const float r1 = rs - (float)h0;
+    const _Float16 h1 = (_Float16)r1;
+    const _Float16 h2 = (_Float16)(r1 - (float)h1);
+    if (g == 0) {
+      corr_q[0] = pack_h2(-(float)h0, -(float)h1);
+      corr_q[1] = pack_h2(-(float)h2, 0.f);
+    }
+  }
+  const float a_s = a.sm_scale_log2;
+
+  // ---- tile copies: codes through a per-lane offset table; scale and zero point one dword per key
+  // (sub-dword direct loads write lane l's zero-extended value to the dword at 4*l)
+  Copy cp;
+  cp.init((unsigned)a.scn, lane);
+  auto issue = [&](int i) {   // own tile i -> ring slot i % NBUF
+    const int t = wave + 4 * i;
+    unsigned char *slot = ring + (i % SKV_NBUF) * SM::SLOT;
+    const int rows = min(SKV_TILE, a.Nk - t * SKV_TILE);
+    // rows past the end read as zero (exact bounds); their scores are masked
+    const rsrc_t rs_k = make_rsrc(codes_bh + (int64_t)t * SKV_TILE * a.scn, (unsigned)((rows - 1) * (int)a.scn + D));
+#pragma unroll
+    for (int c = 0; c < Copy::N; ++c) cp.issue_one(rs_k, slot, 0, lane, c);
+    const rsrc_t rs_s = make_rsrc(reinterpret_cast<const S *>(a.scale) + tk0 + (int64_t)t * SKV_TILE,
+                                  (unsigned)rows * (unsigned)sizeof(S));
+    const rsrc_t rs_z = make_rsrc(a.zp + tk0 + (int64_t)t * SKV_TILE, (unsigned)rows);
+    if (lane < SKV_TILE) {
+      if constexpr (sizeof(S) == 4)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_s, (lptr_t)(slot + SM::K_BYTES), 4, lane * 4, 0, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_s, (lptr_t)(slot + SM::K_BYTES), 2, lane * 2, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_z, (lptr_t)(slot + SM::K_BYTES + SKV_TILE * 4), 1, lane, 0, 0, 0);
+    }
+  };
+  auto scale_of = [](unsigned w) -> float {
+    return std::is_same<S, float>::value ? __builtin_bit_cast(float, w) : lo_to_f32<T>(w);
+  };
+
+  // ---- per-lane read offsets inside a tile
+  const int k_off = lr * D;
+  const int k_swz = KSW::swz(lr);
+  // transposing reads: source lane s of a 16-lane group G addresses 8 bytes of key list[g][s/2] at
+  // d = 32db + 16(G%2) + 8(s%2);  list[g] = {16hh + 4g + 0..3, 16hh + 8 + 4g + 0..3}, the keys whose
+  // probabilities sit in k-group g of the P operand.
+  unsigned vt_off[2][DB];
+  {
+    const int s = lane % 16, G = lane / 16, j = s / 2;
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      const int key = 16 * hh + (j < 4 ? 4 * g + j : 8 + 4 * g + (j - 4));
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+        vt_off[hh][db] = lds_addr(smem) + key * D + (((2 * db + G % 2) ^ KSW::swz(key)) << 4) + 8 * (s % 2);
+    }
+  }
+
+  f32x16 oacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) oacc[db][v] = 0.f;
+  float m_ref = -INFINITY, m_bound = -INFINITY, nm = 0.f, l_run = 0.f, w_run = 0.f;
+  const float thr = SKV_RESCALE_THRESHOLD / a_s;
+
+  auto tile = [&](int i, auto masked_tag) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    const int slot_off = wave * SM::WAVE + (i % SKV_NBUF) * SM::SLOT;
+    const unsigned char *slot = smem + slot_off;
+    const unsigned *skp = reinterpret_cast<const unsigned *>(slot + SM::K_BYTES);
+    const unsigned *zpp = skp + SKV_TILE;
+    const int j0 = (wave + 4 * i) * SKV_TILE;
+    // ---- code rows for the scores (plain reads), then the transposed fragments for P.V (asynchronous)
+    u32x4 kw[D / 32];
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j)
+      kw[j] = *reinterpret_cast<const u32x4 *>(slot + k_off + (((2 * j + g) ^ k_swz) << 4));
+    const unsigned zmine = zpp[lr];
+    // ---- scores: S^T = (1152 + codes) . Q^T, offset removed by the rank-1 MFMA
+    f32x16 f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) f[v] = 0.f;
+#pragma unroll
+    for (int j = 0; j < D / 32; ++j) {
+      f = mfma_h(expand_codes(kw[j][0], kw[j][1]), qf[2 * j], f);
+      f = mfma_h(expand_codes(kw[j][2], kw[j][3]), qf[2 * j + 1], f);
+    }
+    {
+      const unsigned cz = magic_zp_pair(zmine, zmine);      // binary16 pair of 1152 + zp
+      u32x4 corr_k = {0u, 0u, 0u, 0u};
+      if (g == 0) {
+        corr_k[0] = cz;
+        corr_k[1] = cz & 0xffffu;
+      }
+      f = mfma_h(corr_k, corr_q, f);
+    }
+    u32x2 vr[2][DB];
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) vr[hh][db] = lds_read_tr8_async(vt_off[hh][db] + slot_off);
+    // ---- scale, running maximum
+    float mt0 = -INFINITY, mt1 = -INFINITY;
+#pragma unroll
+    for (int aa = 0; aa < 4; ++aa) {
+      const u32x4 sk4 = *reinterpret_cast<const u32x4 *>(skp + 8 * aa + 4 * g);
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) {
+        float uu = f[4 * aa + bb] * scale_of(sk4[bb]);
+        if (MASKED && j0 + 8 * aa + 4 * g + bb >= a.Nk) uu = -INFINITY;
+        f[4 * aa + bb] = uu;
+        if (aa & 1) mt1 = fmaxf(mt1, uu); else mt0 = fmaxf(mt0, uu);
+      }
+    }
+    const float mt = max_across_halves(fmaxf(mt0, mt1));
+    if (__builtin_amdgcn_ballot_w64(mt > m_bound) != 0) {
+      const float m_new = fmaxf(m_ref, mt);
+      const float alpha = m_new == m_ref ? 1.0f : __builtin_amdgcn_exp2f(a_s * (m_ref - m_new));
+      m_ref = m_new;
+      m_bound = m_new + thr;
+      nm = -a_s * m_new;
+      l_run *= alpha;
+      w_run *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) oacc[db][v] *= alpha;
+    }
+    // ---- p = exp2(.);  p' = p * scale_j rounded to binary16;  row sum of p;  offset term of p'
+    u32x4 pf[2];
+#pragma unroll
+    for (int aa = 0; aa < 4; ++aa) {
+      const u32x4 sk4 = *reinterpret_cast<const u32x4 *>(skp + 8 * aa + 4 * g);
+      const u32x4 zk4 = *reinterpret_cast<const u32x4 *>(zpp + 8 * aa + 4 * g);
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int v0 = 4 * aa + 2 * e;
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(a_s, f[v0], nm));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(a_s, f[v0 + 1], nm));
+        l_run += p0 + p1;
+        const unsigned pp = pack_h2(p0 * scale_of(sk4[2 * e]), p1 * scale_of(sk4[2 * e + 1]));
+        pf[aa / 2][2 * (aa % 2) + e] = pp;
+        const unsigned cpair = magic_zp_pair(zk4[2 * e], zk4[2 * e + 1]);
+        w_run = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pp), __builtin_bit_cast(f16x2, cpair), w_run, false);
+      }
+    }
+    // ---- O^T += (1152 + codes)^T . P'^T
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        u32x2 w = vr[hh][db];
+        asm volatile("" : "+v"(w));   // consumers stay behind the wait above
+        oacc[db] = mfma_h(expand_codes(w[0], w[1]), pf[hh], oacc[db]);
+      }
+  };
+
+  // ---- ring: NBUF-1 tiles in flight ahead of the one in work
+#pragma unroll
+  for (int i = 0; i < SKV_NBUF - 1; ++i)
+    if (i < my_tiles) issue(i);
+  for (int i = 0; i < my_tiles; ++i) {
+    if (i + SKV_NBUF - 1 < my_tiles) {
+      issue(i + SKV_NBUF - 1);
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SKV_NBUF - 1) * OPS) : "memory");   // all but the newest NBUF-1 tiles
+    } else {
+      dma_wait();
+    }
+    if ((wave + 4 * i + 1) * SKV_TILE > a.Nk) tile(i, std::true_type{});
+    else tile(i, std::false_type{});
+  }
+
+  // ---- merge the four partial results (waves 1..3 -> LDS -> wave 0)
+  const float l_tot = l_run + swap32_f(l_run);
+  const float w_tot = w_run + swap32_f(w_run);
+  __syncthreads();   // every ring is done with: the merge area overlays them
+  float *mg = reinterpret_cast<float *>(smem);
+  constexpr int MG = SM::MG;
+  if (wave > 0) {
+    float *dst = mg + (wave - 1) * MG;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int d = 32 * db + 8 * (v / 4) + 4 * g + v % 4;
+        dst[d * 32 + lr] = oacc[db][v] - w_tot;   // offset term removed
+      }
+    if (g == 0) {
+      dst[32 * D + lr] = m_ref;
+      dst[32 * D + 32 + lr] = l_tot;
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    float m_all = m_ref;   // finite: wave 0 always owns tile 0
+#pragma unroll
+    for (int w = 0; w < 3; ++w) m_all = fmaxf(m_all, mg[w * MG + 32 * D + lr]);
+    const float s0 = __builtin_amdgcn_exp2f(a_s * (m_ref - m_all));
+    float l_all = l_tot * s0;
+    float sw[3];
+#pragma unroll
+    for (int w = 0; w < 3; ++w) {
+      const float mw = mg[w * MG + 32 * D + lr];   // -inf for a wave without tiles: weight 0
+      sw[w] = __builtin_amdgcn_exp2f(a_s * (mw - m_all));
+      l_all += mg[w * MG + 32 * D + 32 + lr] * sw[w];
+    }
+    const float inv = 1.0f / l_all;
+    if (qi < a.Nq) {
+      T *orow = reinterpret_cast<T *>(a.o) + b * a.sob + h * a.soh + (int64_t)qi * a.son;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int aa = 0; aa < 4; ++aa) {
+          float r[4];
+#pragma unroll
+          for (int bb = 0; bb < 4; ++bb) {
+            const int v = 4 * aa + bb, d = 32 * db + 8 * aa + 4 * g + bb;
+            float acc = (oacc[db][v] - w_tot) * s0;
+#pragma unroll
+            for (int w = 0; w < 3; ++w) acc += mg[w * MG + d * 32 + lr] * sw[w];
+            r[bb] = acc * inv;
+          }
+          u32x2 o2;
+          o2[0] = pack2<T>(r[0], r[1]);
+          o2[1] = pack2<T>(r[2], r[3]);
+          *reinterpret_cast<u32x2 *>(orow + 32 * db + 8 * aa + 4 * g) = o2;
+        }
+      if (g == 0) a.lse[tq0 + qi] = (a_s * m_all + __log2f(l_all)) * kLn2;
+    }
+  }
+}
+
+template <typename T, typename S, int D> static int launch_skv_fwd_tsd(const SkvAttnArgs &x, hipStream_t st) {
+  SkvArgs a;
+  a.q = x.q; a.codes = x.codes; a.scale = x.scale; a.zp = x.zp; a.o = x.o; a.lse = x.lse;
+  a.H = x.H; a.Nq = (int)x.Nq; a.Nk = (int)x.Nk;
+  a.sqb = x.sqb; a.sqh = x.sqh; a.sqn = x.sqn; a.scb = x.scb; a.sch = x.sch; a.scn = x.scn;
+  a.sob = x.sob; a.soh = x.soh; a.son = x.son;
+  a.sm_scale_log2 = x.sm_scale * kLog2e;
+  a.qblocks = (int)((x.Nq + 31) / 32);
+  const int64_t total = (int64_t)a.qblocks * x.B * x.H;
+  if (total > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "attn_fwd_shared_kv: too many query blocks for one launch");
+  skv_fwd_kernel<T, S, D><<<dim3((unsigned)total), dim3(256), 0, st>>>(a);
+  return check_launch("qfa_attn_fwd_shared_kv");
+}
+
+template <typename T, int D> static int launch_skv_fwd_td(const SkvAttnArgs &x, hipStream_t st) {
+  if (x.scale_dtype == QFA_F32) return launch_skv_fwd_tsd<T, float, D>(x, st);
+  return launch_skv_fwd_tsd<T, T, D>(x, st);   // validated: scale_dtype == io_dtype
+}
+
+int launch_skv_fwd(const SkvAttnArgs &x, hipStream_t st) {
+  if (x.io_dtype == QFA_F16) {
+    if (x.D == 128) return launch_skv_fwd_td<_Float16, 128>(x, st);
+    if (x.D == 64) return launch_skv_fwd_td<_Float16, 64>(x, st);
+  } else {
+    if (x.D == 128) return launch_skv_fwd_td<__bf16, 128>(x, st);
+    if (x.D == 64) return launch_skv_fwd_td<__bf16, 64>(x, st);
+  }
+  return set_error(QFA_EUNSUPPORTED, "attn_fwd_shared_kv: head_dim must be 64 or 128");
+}
+
+}  // namespace qfa

@@ -117,6 +117,43 @@ def attn_bwd_quantized(qq: QuantizedTokens, kq: QuantizedTokens, v: torch.Tensor
     return dq, dk, dv
 
 
+# Longest query block the shared-KV kernel is used for: it re-reads the codes once per 32 queries,
+# which pays while the operator is bound by streaming them (the reference's decode-like shapes).
+SHARED_KV_MAX_Q = 128
+
+
+def attn_fwd_shared_kv(q: torch.Tensor, codes: torch.Tensor, scale: torch.Tensor, zero_point: torch.Tensor,
+                       sm_scale: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """O, LSE = attention(q, kv, kv) with kv = (codes - zero_point) * scale, q in fp16 / bf16 and NOT
+    quantized -- the computation of _attn_fwd_kernel_quantized (quant_flash_attn.py:22-83).
+    O has q's dtype; LSE is fp32 [B,H,Nq] (natural log, :79)."""
+    if q.dtype not in _IO_DTYPES:
+        raise TypeError(f"q must be bfloat16 or float16, got {q.dtype}")
+    if codes.dim() != 4 or codes.dtype != torch.int8:
+        raise ValueError("codes must be a 4-D int8 tensor")
+    _lib.require_gpu(q, codes, scale, zero_point)
+    B, H, Nq, D = q.shape
+    Nk = codes.shape[2]
+    if codes.shape != (B, H, Nk, D):
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)}, codes {tuple(codes.shape)}")
+    n = B * H * Nk
+    if scale.dtype != torch.float32 and scale.dtype != q.dtype:
+        scale = scale.to(torch.float32)
+    scale = _flat(scale, scale.dtype, n, "scale")
+    zero_point = _flat(zero_point, torch.int8, n, "zero_point")
+    q, codes = _rows16(q), _rows16(codes)
+    o = torch.empty((B, H, Nq, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, Nq), dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        code = _lib.lib().qfa_attn_fwd_shared_kv(
+            q.data_ptr(), codes.data_ptr(), scale.data_ptr(), _lib.DTYPE_CODE[scale.dtype], zero_point.data_ptr(),
+            o.data_ptr(), lse.data_ptr(), _lib.DTYPE_CODE[q.dtype], B, H, Nq, Nk, D,
+            q.stride(0), q.stride(1), q.stride(2), codes.stride(0), codes.stride(1), codes.stride(2),
+            o.stride(0), o.stride(1), o.stride(2), float(sm_scale), _lib.stream_of(q))
+    _lib.check(code, "qfa_attn_fwd_shared_kv")
+    return o, lse
+
+
 def _io_dtype(t: torch.Tensor) -> torch.dtype:
     return t.dtype if t.dtype in _IO_DTYPES else torch.bfloat16
 

@@ -1,0 +1,95 @@
+"""GPU parity of the shared-KV kernels (the reference's own operator: one quantized tensor serves
+as K and V, Q stays in 16-bit float, quant_flash_attn.py:22-83) against the CPU oracle's literal
+restatement in fp64.  Tolerances: O max-abs <= 2e-2 * max(1, max|O_ref|) and cosine >= 0.999, LSE
+to 2^-8.  (V is the K tensor here, so with outlier channels |O| reaches ~60 and the rounding of a
+16-bit output alone is 2^-11 of that; the bound scales with the largest reference value as it does
+for the gradients.)"""
+import math
+
+import pytest
+import torch
+
+from helpers import assert_close, max_abs
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+LSE_TOL = 2.0 ** -8
+
+
+def _inputs(config, B, H, Nq, Nk, D, dtype, seed):
+    N = max(Nq, Nk)
+    q, k, _, _ = oracle.make_inputs(config, B, H, N, D, seed=seed, dtype=dtype)
+    return q[:, :, :Nq].contiguous(), k[:, :, :Nk].contiguous()
+
+
+CASES = [
+    # B, H, Nq, Nk, D, config, dtype, scale dtype
+    (1, 2, 16, 32, 128, "normal", torch.float16, torch.float16),      # one tile, one wave busy
+    (1, 2, 16, 128, 128, "normal", torch.float16, torch.float16),     # one tile per wave
+    (2, 3, 16, 3000, 128, "normal", torch.float16, torch.float16),    # reference benchmark shape (compute_flops.py:96)
+    (2, 3, 16, 3000, 64, "offset", torch.float16, torch.float16),
+    (1, 2, 1, 1, 128, "normal", torch.float16, torch.float16),        # single query, single key
+    (1, 2, 5, 33, 64, "uniform", torch.float16, torch.float32),       # ragged tail of one key
+    (2, 2, 97, 689, 128, "offset", torch.bfloat16, torch.float32),    # four query blocks, ragged both ways
+    (1, 2, 17, 1023, 128, "outlier", torch.float16, torch.float16),
+    (1, 4, 32, 512, 64, "normal", torch.bfloat16, torch.bfloat16),
+    (1, 2, 128, 4096, 128, "normal", torch.bfloat16, torch.float16),  # scale converted by the wrapper
+]
+
+
+@pytest.mark.parametrize("B,H,Nq,Nk,D,config,dtype,sdtype", CASES)
+def test_shared_kv_forward_vs_oracle(qfa, B, H, Nq, Nk, D, config, dtype, sdtype):
+    q, kv = _inputs(config, B, H, Nq, Nk, D, dtype, seed=Nq + Nk + D)
+    sm = 1.0 / math.sqrt(D)
+    codes, scale, zp = qfa.asymmetric_quant_per_token(kv.to(DEV), scale_dtype=sdtype)
+    o, lse = qfa.attn_fwd_shared_kv(q.to(DEV), codes, scale, zp, sm)
+    torch.cuda.synchronize()
+    o_ref, lse_ref = oracle.legacy_fwd(q, codes.cpu(), scale.cpu(), zp.cpu(), sm)
+    assert o.dtype == dtype and o.shape == (B, H, Nq, D) and lse.shape == (B, H, Nq)
+    assert_close("O", o.cpu(), o_ref, scaled=True)
+    assert max_abs(lse.cpu(), lse_ref) < LSE_TOL
+
+
+def test_shared_kv_offsets_cancel(qfa):
+    """Every token with the same nonzero codes and extreme zero points: the 1152-offset terms the
+    kernel adds to make the codes binary16 operands are orders of magnitude above the result and
+    must cancel exactly.  O = the common dequantized row, whatever the softmax weights."""
+    B, H, Nq, Nk, D = 1, 2, 16, 96, 128
+    g = torch.Generator().manual_seed(5)
+    row = torch.randint(-128, 128, (1, 1, 1, D), generator=g, dtype=torch.int32).to(torch.int8)
+    codes = row.expand(B, H, Nk, D).contiguous()
+    zp = torch.full((B, H, Nk, 1), -128, dtype=torch.int8)
+    scale = torch.full((B, H, Nk, 1), 0.03125, dtype=torch.float16)
+    q = torch.randn((B, H, Nq, D), generator=g).to(torch.float16)
+    o, lse = qfa.attn_fwd_shared_kv(q.to(DEV), codes.to(DEV), scale.to(DEV), zp.to(DEV), 0.1)
+    want = ((row.double() + 128.0) * 0.03125).expand(B, H, Nq, D)
+    assert max_abs(o.cpu(), want) <= 2.0 ** -9 * float(want.abs().max())   # one fp16 rounding of the output
+    o_ref, lse_ref = oracle.legacy_fwd(q, codes, scale, zp, 0.1)
+    assert max_abs(lse.cpu(), lse_ref) < LSE_TOL
+
+
+def test_shared_kv_strided_views(qfa):
+    """q and the codes handed over as views of larger buffers (token stride > D)."""
+    B, H, Nq, Nk, D = 2, 2, 16, 200, 64
+    q, kv = _inputs("normal", B, H, Nq, Nk, D, torch.float16, seed=9)
+    sm = 0.125
+    codes, scale, zp = qfa.asymmetric_quant_per_token(kv.to(DEV))
+    big_c = torch.zeros((B, H, Nk, 2 * D), dtype=torch.int8, device=DEV)
+    big_c[..., :D] = codes
+    big_q = torch.zeros((B, H, Nq, 3 * D), dtype=torch.float16, device=DEV)
+    big_q[..., D:2 * D] = q.to(DEV)
+    o1, l1 = qfa.attn_fwd_shared_kv(q.to(DEV), codes, scale, zp, sm)
+    o2, l2 = qfa.attn_fwd_shared_kv(big_q[..., D:2 * D], big_c[..., :D], scale, zp, sm)
+    assert torch.equal(o1, o2) and torch.equal(l1, l2)
+
+
+def test_shared_kv_rejects_bad_arguments(qfa):
+    q = torch.zeros((1, 1, 16, 96), dtype=torch.float16, device=DEV)
+    codes = torch.zeros((1, 1, 64, 96), dtype=torch.int8, device=DEV)
+    scale = torch.ones((1, 1, 64, 1), dtype=torch.float16, device=DEV)
+    zp = torch.zeros((1, 1, 64, 1), dtype=torch.int8, device=DEV)
+    with pytest.raises(RuntimeError, match="head_dim"):
+        qfa.attn_fwd_shared_kv(q, codes, scale, zp, 0.1)
+    with pytest.raises(TypeError):
+        qfa.attn_fwd_shared_kv(q.float(), codes, scale, zp, 0.1)
