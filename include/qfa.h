@@ -92,6 +92,28 @@ int qfa_attn_fwd(const int8_t *qc, const float *sq, const int8_t *zq, const int3
                  int64_t sob, int64_t soh, int64_t son, float sm_scale, int causal, void *stream);
 
 /*
+ * Attention forward of the reference's own operator, for short query blocks:
+ *     O = softmax(sm_scale * Q KV^T) KV,   KV = scale * (codes - zp) per token,   LSE = logsumexp
+ * One quantized tensor serves as K and V and Q stays in 16-bit float, exactly as in
+ * _attn_fwd_kernel_quantized (quant_flash_attn.py:22-83; launched from :178-204 with one program
+ * per (batch, head) and the whole query block in it).  The kernel streams the INT8 codes once per
+ * block of 32 queries and feeds them to the 16-bit MFMAs as exact binary16 integers, so it is bound
+ * by reading the codes; it is the right entry point while Nq is small against Nk (decoding, the
+ * reference's benchmark shape Nq=16, Nk=3000 of compute_flops.py:96).  For long query blocks
+ * qfa_attn_fwd (quantized Q, INT8 MFMA) is the faster path.
+ *   q, o   [B,H,Nq,D] of io_dtype (QFA_F16 or QFA_BF16; bf16 queries enter the products rounded
+ *          to binary16), strides sq?, so?;  lse float [B*H*Nq]
+ *   codes  int8 [B,H,Nk,D], strides sc?;  zp int8 [B*H*Nk]
+ *   scale  [B*H*Nk] of scale_dtype: QFA_F32, or the same 16-bit type as io_dtype
+ *   D in {64, 128}.  q, codes, o 16-byte aligned, strides multiples of 16 bytes, scn < 2^23.
+ *   The sum of a query's D elements must stay inside binary16 range (|sum| < 65504).
+ */
+int qfa_attn_fwd_shared_kv(const void *q, const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp,
+                           void *o, float *lse, int io_dtype, int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D,
+                           int64_t sqb, int64_t sqh, int64_t sqn, int64_t scb, int64_t sch, int64_t scn, int64_t sob,
+                           int64_t soh, int64_t son, float sm_scale, void *stream);
+
+/*
  * Measurement hook, same arguments as qfa_attn_fwd: runs the forward kernel with the exponentials
  * and the P.V product compiled out (same K/V/Q loads, INT8 QK^T MFMAs, zero-point correction, key
  * scaling and running row maximum).  O is left untouched; lse receives the scaled row maxima.

@@ -10,8 +10,10 @@ Two autograd entry points, both backed by the HIP kernels behind qfa_attn_fwd / 
   QuantFlashAttention.apply(q, kv_fp16, kv_quant, sm_scale)     (alias quant_flash_attn)
       The reference's own entry point (quant_flash_attn.py:173-240): one quantized tensor serves as
       K and V, `kv_fp16` only receives the gradient, backward returns (dq, dkv, None, None) with
-      dkv = dK + dV (:161).  Difference from the reference, stated: Q is quantized per token too
-      (the reference keeps Q in fp16), because the score product runs on INT8 MFMA.
+      dkv = dK + dV (:161).  Query blocks of up to SHARED_KV_MAX_Q tokens run the reference's
+      computation itself in the forward (Q in 16-bit, qfa_attn_fwd_shared_kv).  Longer ones, and
+      the backward, go through the INT8-score kernels, where Q is quantized per token too (stated
+      difference from the reference, which keeps Q in fp16).
 """
 from __future__ import annotations
 
@@ -206,26 +208,40 @@ class QuantFlashAttention(torch.autograd.Function):
         _lib.require_gpu(q, codes, scale, zp)
         if q.dim() != 4 or codes.shape != kv_fp16.shape or q.shape[-1] != codes.shape[-1]:
             raise ValueError(f"shape mismatch: q {tuple(q.shape)}, kv {tuple(kv_fp16.shape)}, codes {tuple(codes.shape)}")
-        io = _io_dtype(q)
-        qq = quantize_for_attention(q)
-        # K operand: the caller's codes with the scale exactly as stored (fp16 in the reference)
-        kq = QuantizedTokens(codes, scale.to(torch.float32), zp,
-                             codes.sum(dim=-1, keepdim=True, dtype=torch.int32))
-        v16 = dequantize_per_token(codes, scale, zp, io)          # V operand: dequant(kv) (:65)
-        o, lse = attn_fwd_quantized(qq, kq, v16, False, sm_scale)
-        ctx.save_for_backward(*qq, *kq, v16, o, lse)
         ctx.sm_scale = float(sm_scale)
         ctx.q_dtype, ctx.kv_dtype = q.dtype, kv_fp16.dtype
+        ctx.shared_kv = q.shape[2] <= SHARED_KV_MAX_Q and q.dtype in _IO_DTYPES
+        if ctx.shared_kv:
+            # the reference's computation itself: Q unquantized, the codes streamed once (:50-69)
+            o, lse = attn_fwd_shared_kv(q, codes, scale, zp, sm_scale)
+            ctx.save_for_backward(q, codes, scale, zp, o, lse)
+            return o
+        io = _io_dtype(q)
+        qq, kq, v16 = _legacy_operands(q, codes, scale, zp, io)
+        o, lse = attn_fwd_quantized(qq, kq, v16, False, sm_scale)
+        ctx.save_for_backward(*qq, *kq, v16, o, lse)
         return o.to(q.dtype)
 
     @staticmethod
     def backward(ctx, grad_output):
         t = ctx.saved_tensors
-        qq, kq = QuantizedTokens(*t[0:4]), QuantizedTokens(*t[4:8])
-        v16, o, lse = t[8], t[9], t[10]
+        if ctx.shared_kv:
+            q, codes, scale, zp, o, lse = t
+            qq, kq, v16 = _legacy_operands(q, codes, scale, zp, q.dtype)
+        else:
+            qq, kq = QuantizedTokens(*t[0:4]), QuantizedTokens(*t[4:8])
+            v16, o, lse = t[8], t[9], t[10]
         dq, dk, dv = attn_bwd_quantized(qq, kq, v16, o, grad_output.to(v16.dtype), lse, False, ctx.sm_scale)
         dkv = dk.to(torch.float32).add_(dv).to(ctx.kv_dtype)      # :161 (dk already carries sm_scale)
         return dq.to(ctx.q_dtype), dkv, None, None
+
+
+def _legacy_operands(q, codes, scale, zp, io):
+    """Operands of the INT8-score kernels for the reference's entry point: Q quantized per token,
+    K = the caller's codes with the scale exactly as stored, V = dequant(kv) (quant_flash_attn.py:65)."""
+    qq = quantize_for_attention(q)
+    kq = QuantizedTokens(codes, scale.to(torch.float32), zp, codes.sum(dim=-1, keepdim=True, dtype=torch.int32))
+    return qq, kq, dequantize_per_token(codes, scale, zp, io)
 
 
 quant_flash_attn = QuantFlashAttention.apply
