@@ -114,6 +114,25 @@ int qfa_attn_fwd_shared_kv(const void *q, const int8_t *codes, const void *scale
                            int64_t soh, int64_t son, float sm_scale, void *stream);
 
 /*
+ * Backward of qfa_attn_fwd_shared_kv for one short query block (Nq <= 32), fp16:
+ *     P = exp(sm_scale Q KV^T - LSE),  dP = dO KV^T,  dS = sm_scale P o (dP - delta),  delta = rowsum(O o dO)
+ *     dQ = dS KV,    dKV = P^T dO + dS^T Q
+ * Replaces the launches made by QuantFlashAttention.backward (quant_flash_attn.py:207-237):
+ * _bwd_preprocess_kernel (:87-101; delta is computed inside) and _attn_bwd_kernel_quantized
+ * (:104-166), which also stores the single gradient dKV = dV + dK (:161).  One workgroup per
+ * (batch, head) streams the codes once and writes each dKV row once.
+ *   q, o, dout, dq [B,H,Nq,D] and dkv [B,H,Nk,D] fp16 (io_dtype must be QFA_F16), strides as given;
+ *   codes, scale, scale_dtype, zp, lse as in the forward.  D in {64, 128}.
+ *   The sums of a query's and of a dO row's D elements must stay inside binary16 range.
+ */
+int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp,
+                           const void *o, const void *dout, const float *lse, void *dq, void *dkv, int io_dtype,
+                           int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D, int64_t sqb, int64_t sqh, int64_t sqn,
+                           int64_t scb, int64_t sch, int64_t scn, int64_t sob, int64_t soh, int64_t son, int64_t sdob,
+                           int64_t sdoh, int64_t sdon, int64_t sdqb, int64_t sdqh, int64_t sdqn, int64_t sdkb,
+                           int64_t sdkh, int64_t sdkn, float sm_scale, void *stream);
+
+/*
  * Measurement hook, same arguments as qfa_attn_fwd: runs the forward kernel with the exponentials
  * and the P.V product compiled out (same K/V/Q loads, INT8 QK^T MFMAs, zero-point correction, key
  * scaling and running row maximum).  O is left untouched; lse receives the scaled row maxima.

@@ -12,12 +12,12 @@ GPU only: a CPU tensor or a missing libqfa.so raises; there is no fallback imple
 from .asymmetric_quant import (QuantizedTokens, asymmetric_quant_per_token, dequantize_per_token,
                                quantize_for_attention)
 from .quant_flash_attn import (QuantFlashAttention, QuantFlashAttnQKV, attn_bwd_quantized, attn_fwd_quantized,
-                               attn_fwd_shared_kv,
+                               attn_bwd_shared_kv, attn_fwd_shared_kv,
                                quant_flash_attn, quant_flash_attn_qkv)
 
 __all__ = [
     "QuantizedTokens", "asymmetric_quant_per_token", "dequantize_per_token", "quantize_for_attention",
     "QuantFlashAttention", "QuantFlashAttnQKV", "quant_flash_attn", "quant_flash_attn_qkv",
-    "attn_fwd_quantized", "attn_bwd_quantized", "attn_fwd_shared_kv",
+    "attn_fwd_quantized", "attn_bwd_quantized", "attn_fwd_shared_kv", "attn_bwd_shared_kv",
 ]
 __version__ = "0.1.0"

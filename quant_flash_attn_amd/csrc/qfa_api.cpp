@@ -120,33 +120,65 @@ int qfa_attn_fwd(const int8_t *qc, const float *sq, const int8_t *zq, const int3
   return launch_fwd(a, (hipStream_t)stream);
 }
 
+static int check_shared_kv(const char *who, const SkvAttnArgs &a) {
+  if (!a.q || !a.codes || !a.scale || !a.zp || !a.o || !a.lse) return set_error(QFA_EINVAL, "%s: null pointer argument", who);
+  if (a.io_dtype != QFA_BF16 && a.io_dtype != QFA_F16)
+    return set_error(QFA_EINVAL, "%s: io_dtype must be QFA_BF16 or QFA_F16", who);
+  if (a.scale_dtype != QFA_F32 && a.scale_dtype != a.io_dtype)
+    return set_error(QFA_EINVAL, "%s: scale_dtype must be QFA_F32 or equal to io_dtype", who);
+  if (a.B <= 0 || a.H <= 0 || a.Nq <= 0 || a.Nk <= 0) return set_error(QFA_EINVAL, "%s: B, H, Nq, Nk must be positive", who);
+  if (a.Nq > 0x7fffff00LL || a.Nk > 0x7fffff00LL) return set_error(QFA_EUNSUPPORTED, "%s: sequence too long", who);
+  if (a.D != 64 && a.D != 128) return set_error(QFA_EUNSUPPORTED, "%s: head_dim %d not in {64, 128}", who, a.D);
+  if (!(a.sm_scale > 0.0f) || !(a.sm_scale < 3.0e38f))
+    return set_error(QFA_EINVAL, "%s: sm_scale must be a positive finite number", who);
+  if (!aligned16(a.q) || !aligned16(a.codes) || !aligned16(a.o))
+    return set_error(QFA_EINVAL, "%s: q, codes, o must be 16-byte aligned", who);
+  if (!strides_ok(a.sqb, a.sqh, a.sqn, a.D, 2) || !strides_ok(a.scb, a.sch, a.scn, a.D, 1) ||
+      !strides_ok(a.sob, a.soh, a.son, a.D, 2))
+    return set_error(QFA_EINVAL, "%s: strides must be positive multiples of 16 bytes, token stride >= D", who);
+  if (a.scn >= (1 << 23)) return set_error(QFA_EUNSUPPORTED, "%s: token strides of 2^23 elements or more are not supported", who);
+  return 0;
+}
+
 int qfa_attn_fwd_shared_kv(const void *q, const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp,
                            void *o, float *lse, int io_dtype, int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D,
                            int64_t sqb, int64_t sqh, int64_t sqn, int64_t scb, int64_t sch, int64_t scn, int64_t sob,
                            int64_t soh, int64_t son, float sm_scale, void *stream) {
-  const char *who = "attn_fwd_shared_kv";
-  if (!q || !codes || !scale || !zp || !o || !lse) return set_error(QFA_EINVAL, "%s: null pointer argument", who);
-  if (io_dtype != QFA_BF16 && io_dtype != QFA_F16)
-    return set_error(QFA_EINVAL, "%s: io_dtype must be QFA_BF16 or QFA_F16", who);
-  if (scale_dtype != QFA_F32 && scale_dtype != io_dtype)
-    return set_error(QFA_EINVAL, "%s: scale_dtype must be QFA_F32 or equal to io_dtype", who);
-  if (B <= 0 || H <= 0 || Nq <= 0 || Nk <= 0) return set_error(QFA_EINVAL, "%s: B, H, Nq, Nk must be positive", who);
-  if (Nq > 0x7fffff00LL || Nk > 0x7fffff00LL) return set_error(QFA_EUNSUPPORTED, "%s: sequence too long", who);
-  if (D != 64 && D != 128) return set_error(QFA_EUNSUPPORTED, "%s: head_dim %d not in {64, 128}", who, D);
-  if (!(sm_scale > 0.0f) || !(sm_scale < 3.0e38f))
-    return set_error(QFA_EINVAL, "%s: sm_scale must be a positive finite number", who);
-  if (!aligned16(q) || !aligned16(codes) || !aligned16(o))
-    return set_error(QFA_EINVAL, "%s: q, codes, o must be 16-byte aligned", who);
-  if (!strides_ok(sqb, sqh, sqn, D, 2) || !strides_ok(scb, sch, scn, D, 1) || !strides_ok(sob, soh, son, D, 2))
-    return set_error(QFA_EINVAL, "%s: strides must be positive multiples of 16 bytes, token stride >= D", who);
-  if (scn >= (1 << 23)) return set_error(QFA_EUNSUPPORTED, "%s: token strides of 2^23 elements or more are not supported", who);
   SkvAttnArgs a;
   memset(&a, 0, sizeof(a));
   a.q = q; a.codes = codes; a.scale = scale; a.zp = zp; a.o = o; a.lse = lse;
   a.B = B; a.H = H; a.Nq = Nq; a.Nk = Nk; a.D = D; a.io_dtype = io_dtype; a.scale_dtype = scale_dtype;
   a.sqb = sqb; a.sqh = sqh; a.sqn = sqn; a.scb = scb; a.sch = sch; a.scn = scn; a.sob = sob; a.soh = soh; a.son = son;
   a.sm_scale = sm_scale;
+  if (int e = check_shared_kv("attn_fwd_shared_kv", a)) return e;
   return launch_skv_fwd(a, (hipStream_t)stream);
+}
+
+int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp,
+                           const void *o, const void *dout, const float *lse, void *dq, void *dkv, int io_dtype,
+                           int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D, int64_t sqb, int64_t sqh, int64_t sqn,
+                           int64_t scb, int64_t sch, int64_t scn, int64_t sob, int64_t soh, int64_t son, int64_t sdob,
+                           int64_t sdoh, int64_t sdon, int64_t sdqb, int64_t sdqh, int64_t sdqn, int64_t sdkb,
+                           int64_t sdkh, int64_t sdkn, float sm_scale, void *stream) {
+  const char *who = "attn_bwd_shared_kv";
+  SkvAttnArgs a;
+  memset(&a, 0, sizeof(a));
+  a.q = q; a.codes = codes; a.scale = scale; a.zp = zp; a.o = const_cast<void *>(o); a.lse = const_cast<float *>(lse);
+  a.dout = dout; a.dq = dq; a.dkv = dkv;
+  a.B = B; a.H = H; a.Nq = Nq; a.Nk = Nk; a.D = D; a.io_dtype = io_dtype; a.scale_dtype = scale_dtype;
+  a.sqb = sqb; a.sqh = sqh; a.sqn = sqn; a.scb = scb; a.sch = sch; a.scn = scn; a.sob = sob; a.soh = soh; a.son = son;
+  a.sdob = sdob; a.sdoh = sdoh; a.sdon = sdon; a.sdqb = sdqb; a.sdqh = sdqh; a.sdqn = sdqn;
+  a.sdkb = sdkb; a.sdkh = sdkh; a.sdkn = sdkn;
+  a.sm_scale = sm_scale;
+  if (int e = check_shared_kv(who, a)) return e;
+  if (!dout || !dq || !dkv) return set_error(QFA_EINVAL, "%s: null pointer argument", who);
+  if (io_dtype != QFA_F16) return set_error(QFA_EUNSUPPORTED, "%s: io_dtype must be QFA_F16", who);
+  if (Nq > 32) return set_error(QFA_EUNSUPPORTED, "%s: at most 32 queries per (batch, head), got %lld", who, (long long)Nq);
+  if (!aligned16(dout) || !aligned16(dq) || !aligned16(dkv))
+    return set_error(QFA_EINVAL, "%s: dout, dq, dkv must be 16-byte aligned", who);
+  if (!strides_ok(sdob, sdoh, sdon, D, 2) || !strides_ok(sdqb, sdqh, sdqn, D, 2) || !strides_ok(sdkb, sdkh, sdkn, D, 2))
+    return set_error(QFA_EINVAL, "%s: strides must be positive multiples of 16 bytes, token stride >= D", who);
+  return launch_skv_bwd(a, (hipStream_t)stream);
 }
 
 int qfa_bench_qk_stage(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,

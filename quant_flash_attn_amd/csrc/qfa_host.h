@@ -45,11 +45,14 @@ int64_t bwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D)
 struct SkvAttnArgs {
   const void *q; const int8_t *codes; const void *scale; const int8_t *zp;
   void *o; float *lse;
+  const void *dout; void *dq; void *dkv;   // backward only
   int64_t B, H, Nq, Nk;
   int64_t sqb, sqh, sqn, scb, sch, scn, sob, soh, son;
+  int64_t sdob, sdoh, sdon, sdqb, sdqh, sdqn, sdkb, sdkh, sdkn;
   float sm_scale;
   int D, io_dtype, scale_dtype;
 };
 int launch_skv_fwd(const SkvAttnArgs &a, hipStream_t st);
+int launch_skv_bwd(const SkvAttnArgs &a, hipStream_t st);   // io_dtype QFA_F16, Nq <= 32
 
 }  // namespace qfa

@@ -25,8 +25,8 @@
 // lanes, lane i receives byte i%8 of the 8-byte rows addressed by lanes (i%16)/8 + {0,2,..,14}.
 #include <type_traits>
 
-#include "qfa_device.h"
 #include "qfa_host.h"
+#include "qfa_skv_common.h"
 
 namespace qfa {
 
@@ -40,34 +40,7 @@ struct SkvArgs {
   int qblocks;   // ceil(Nq / 32)
 };
 
-constexpr int SKV_TILE = 32;     // keys per tile
 constexpr int SKV_NBUF = 4;      // ring depth per wave
-constexpr float SKV_RESCALE_THRESHOLD = 4.0f;   // p <= 2^4: p * scale stays inside binary16 for any fp16 K
-
-__device__ __forceinline__ f32x16 mfma_h(u32x4 a, u32x4 b, f32x16 c) { return mfma_16b<_Float16>(a, b, c); }
-// two unsigned bytes (positions A and A+1 of w) -> packed binary16 pair (1024 + byte)
-template <int A> __device__ __forceinline__ unsigned magic_pair(unsigned w) {
-  constexpr unsigned sel = 0x04000400u | (unsigned)A | ((unsigned)(A + 1) << 16);
-  return __builtin_amdgcn_perm(0x64646464u, w, sel);
-}
-// 8 code bytes (two dwords) -> 8 binary16 values 1152 + code
-__device__ __forceinline__ u32x4 expand_codes(unsigned w0, unsigned w1) {
-  w0 ^= 0x80808080u;
-  w1 ^= 0x80808080u;
-  return u32x4{magic_pair<0>(w0), magic_pair<2>(w0), magic_pair<0>(w1), magic_pair<2>(w1)};
-}
-__device__ __forceinline__ unsigned pack_h2(float a, float b) { return pack2<_Float16>(a, b); }
-// binary16 pair (1152 + za, 1152 + zb) from two zero points held in the low bytes of za and zb
-__device__ __forceinline__ unsigned magic_zp_pair(unsigned za, unsigned zb) {
-  return __builtin_amdgcn_perm(za, zb, 0x0c000c04u) ^ 0x64806480u;
-}
-// ds_read_b64_tr_b8, issued like lds_read_tr16_async: invisible to the compiler's wait bookkeeping
-// (which would make it wait for every direct-to-LDS load in flight), to be followed by lds_wait_async.
-__device__ __forceinline__ u32x2 lds_read_tr8_async(unsigned addr) {
-  u32x2 r;
-  asm volatile("ds_read_b64_tr_b8 %0, %1" : "=v"(r) : "v"(addr) : "memory");
-  return r;
-}
 
 template <int D> struct SkvSmem {
   static constexpr int K_BYTES = SKV_TILE * D;             // codes of a tile, rows dense, chunks swizzled (Swz<D>)
@@ -165,15 +138,14 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
   // transposing reads: source lane s of a 16-lane group G addresses 8 bytes of key list[g][s/2] at
   // d = 32db + 16(G%2) + 8(s%2);  list[g] = {16hh + 4g + 0..3, 16hh + 8 + 4g + 0..3}, the keys whose
   // probabilities sit in k-group g of the P operand.
-  unsigned vt_off[2][DB];
+  // (block db enters as an XOR of 2db on the chunk index: smem is aligned to a whole row)
+  unsigned vt_off[2];
   {
     const int s = lane % 16, G = lane / 16, j = s / 2;
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh) {
       const int key = 16 * hh + (j < 4 ? 4 * g + j : 8 + 4 * g + (j - 4));
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-        vt_off[hh][db] = lds_addr(smem) + key * D + (((2 * db + G % 2) ^ KSW::swz(key)) << 4) + 8 * (s % 2);
+      vt_off[hh] = key * D + (((G % 2) ^ KSW::swz(key)) << 4) + 8 * (s % 2);
     }
   }
 
@@ -220,7 +192,7 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
-      for (int db = 0; db < DB; ++db) vr[hh][db] = lds_read_tr8_async(vt_off[hh][db] + slot_off);
+      for (int db = 0; db < DB; ++db) vr[hh][db] = lds_read_tr8_async(lds_addr(smem) + slot_off + (vt_off[hh] ^ ((2 * db) << 4)));
     // ---- scale, running maximum
     float mt0 = -INFINITY, mt1 = -INFINITY;
 #pragma unroll
@@ -267,13 +239,12 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
       }
     }
     // ---- O^T += (1152 + codes)^T . P'^T
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    lds_wait_all();
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        u32x2 w = vr[hh][db];
-        asm volatile("" : "+v"(w));   // consumers stay behind the wait above
+        const u32x2 w = tie(vr[hh][db]);
         oacc[db] = mfma_h(expand_codes(w[0], w[1]), pf[hh], oacc[db]);
       }
   };

@@ -1,0 +1,51 @@
+// Shared pieces of the shared-KV kernels (forward and backward): tile geometry and the helpers that
+// turn INT8 codes into exact binary16 MFMA operands.
+//
+// A code byte c (two's complement) with its top bit flipped is the unsigned byte c + 128; placed
+// under the constant high byte 0x64 it is the binary16 number 1152 + c exactly.  One XOR per dword
+// and one byte permute per pair of elements therefore make a 16-bit MFMA operand out of codes, and
+// the offset 1152 + zero_point is taken out again exactly by the kernels (a rank-1 MFMA update where
+// the codes are contracted over d, a v_dot2 accumulation where they are contracted over tokens).
+#pragma once
+#include "qfa_device.h"
+
+namespace qfa {
+
+constexpr int SKV_TILE = 32;     // keys per tile
+constexpr float SKV_RESCALE_THRESHOLD = 4.0f;   // p <= 2^4: p * scale stays inside binary16 for any fp16 K
+
+__device__ __forceinline__ f32x16 mfma_h(u32x4 a, u32x4 b, f32x16 c) { return mfma_16b<_Float16>(a, b, c); }
+// two unsigned bytes (positions A and A+1 of w) -> packed binary16 pair (1024 + byte)
+template <int A> __device__ __forceinline__ unsigned magic_pair(unsigned w) {
+  constexpr unsigned sel = 0x04000400u | (unsigned)A | ((unsigned)(A + 1) << 16);
+  return __builtin_amdgcn_perm(0x64646464u, w, sel);
+}
+// 8 code bytes (two dwords) -> 8 binary16 values 1152 + code
+__device__ __forceinline__ u32x4 expand_codes(unsigned w0, unsigned w1) {
+  w0 ^= 0x80808080u;
+  w1 ^= 0x80808080u;
+  return u32x4{magic_pair<0>(w0), magic_pair<2>(w0), magic_pair<0>(w1), magic_pair<2>(w1)};
+}
+__device__ __forceinline__ unsigned pack_h2(float a, float b) { return pack2<_Float16>(a, b); }
+// binary16 pair (1152 + za, 1152 + zb) from two zero points held in the low bytes of za and zb
+__device__ __forceinline__ unsigned magic_zp_pair(unsigned za, unsigned zb) {
+  return __builtin_amdgcn_perm(za, zb, 0x0c000c04u) ^ 0x64806480u;
+}
+// ds_read_b64_tr_b8, issued like lds_read_tr16_async: invisible to the compiler's wait bookkeeping
+// (which would make it wait for every direct-to-LDS load in flight); use the result only after
+// lds_wait_all() and through tie().
+__device__ __forceinline__ u32x2 lds_read_tr8_async(unsigned addr) {
+  u32x2 r;
+  asm volatile("ds_read_b64_tr_b8 %0, %1" : "=v"(r) : "v"(addr) : "memory");
+  return r;
+}
+
+// wait for every LDS operation of this wave; `tie` keeps the users of an asynchronously loaded
+// register pair behind the wait that precedes it in program order
+__device__ __forceinline__ void lds_wait_all() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ u32x2 tie(u32x2 w) {
+  asm volatile("" : "+v"(w));
+  return w;
+}
+
+}  // namespace qfa

@@ -11,8 +11,9 @@ Two autograd entry points, both backed by the HIP kernels behind qfa_attn_fwd / 
       The reference's own entry point (quant_flash_attn.py:173-240): one quantized tensor serves as
       K and V, `kv_fp16` only receives the gradient, backward returns (dq, dkv, None, None) with
       dkv = dK + dV (:161).  Query blocks of up to SHARED_KV_MAX_Q tokens run the reference's
-      computation itself in the forward (Q in 16-bit, qfa_attn_fwd_shared_kv).  Longer ones, and
-      the backward, go through the INT8-score kernels, where Q is quantized per token too (stated
+      computation itself in the forward (Q in 16-bit, qfa_attn_fwd_shared_kv), and fp16 blocks of
+      up to SHARED_KV_BWD_MAX_Q tokens also in the backward (qfa_attn_bwd_shared_kv).  Everything
+      else goes through the INT8-score kernels, where Q is quantized per token too (stated
       difference from the reference, which keeps Q in fp16).
 """
 from __future__ import annotations
@@ -156,6 +157,45 @@ def attn_fwd_shared_kv(q: torch.Tensor, codes: torch.Tensor, scale: torch.Tensor
     return o, lse
 
 
+# Largest query block of the shared-KV backward kernel (one 32-row MFMA block of queries).
+SHARED_KV_BWD_MAX_Q = 32
+
+
+def attn_bwd_shared_kv(q: torch.Tensor, codes: torch.Tensor, scale: torch.Tensor, zero_point: torch.Tensor,
+                       o: torch.Tensor, do: torch.Tensor, lse: torch.Tensor, sm_scale: float
+                       ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """dQ, dKV of attn_fwd_shared_kv in fp16: the computation of _attn_bwd_kernel_quantized
+    (quant_flash_attn.py:104-166) with dKV = dV + dK as stored there (:161).  q, o, do fp16
+    [B,H,Nq,D] with Nq <= 32; lse as returned by the forward."""
+    if q.dtype != torch.float16 or o.dtype != torch.float16:
+        raise TypeError("the shared-KV backward kernel computes in float16: q and o must be float16")
+    if codes.dim() != 4 or codes.dtype != torch.int8:
+        raise ValueError("codes must be a 4-D int8 tensor")
+    B, H, Nq, D = q.shape
+    Nk = codes.shape[2]
+    if codes.shape != (B, H, Nk, D) or o.shape != q.shape or do.shape != q.shape:
+        raise ValueError("shape mismatch between q / o / do and the codes")
+    do = do.to(torch.float16)
+    _lib.require_gpu(q, codes, scale, zero_point, o, do, lse)
+    n = B * H * Nk
+    if scale.dtype not in (torch.float32, torch.float16):
+        scale = scale.to(torch.float32)
+    scale = _flat(scale, scale.dtype, n, "scale")
+    zero_point = _flat(zero_point, torch.int8, n, "zero_point")
+    lse = _flat(lse, torch.float32, B * H * Nq, "lse")
+    q, codes, o, do = _rows16(q), _rows16(codes), _rows16(o), _rows16(do)
+    dq = torch.empty((B, H, Nq, D), dtype=torch.float16, device=q.device)
+    dkv = torch.empty((B, H, Nk, D), dtype=torch.float16, device=q.device)
+    s = lambda t: (t.stride(0), t.stride(1), t.stride(2))
+    with torch.cuda.device(q.device):
+        code = _lib.lib().qfa_attn_bwd_shared_kv(
+            q.data_ptr(), codes.data_ptr(), scale.data_ptr(), _lib.DTYPE_CODE[scale.dtype], zero_point.data_ptr(),
+            o.data_ptr(), do.data_ptr(), lse.data_ptr(), dq.data_ptr(), dkv.data_ptr(), _lib.QFA_F16,
+            B, H, Nq, Nk, D, *s(q), *s(codes), *s(o), *s(do), *s(dq), *s(dkv), float(sm_scale), _lib.stream_of(q))
+    _lib.check(code, "qfa_attn_bwd_shared_kv")
+    return dq, dkv
+
+
 def _io_dtype(t: torch.Tensor) -> torch.dtype:
     return t.dtype if t.dtype in _IO_DTYPES else torch.bfloat16
 
@@ -227,6 +267,9 @@ class QuantFlashAttention(torch.autograd.Function):
         t = ctx.saved_tensors
         if ctx.shared_kv:
             q, codes, scale, zp, o, lse = t
+            if q.dtype == torch.float16 and q.shape[2] <= SHARED_KV_BWD_MAX_Q:
+                dq, dkv = attn_bwd_shared_kv(q, codes, scale, zp, o, grad_output, lse, ctx.sm_scale)
+                return dq, dkv.to(ctx.kv_dtype), None, None
             qq, kq, v16 = _legacy_operands(q, codes, scale, zp, q.dtype)
         else:
             qq, kq = QuantizedTokens(*t[0:4]), QuantizedTokens(*t[4:8])

@@ -9,7 +9,7 @@ import math
 import pytest
 import torch
 
-from helpers import assert_close, max_abs
+from helpers import COS_TOL, assert_close, max_abs
 from oracle import oracle
 
 pytestmark = pytest.mark.gpu
@@ -49,6 +49,60 @@ def test_shared_kv_forward_vs_oracle(qfa, B, H, Nq, Nk, D, config, dtype, sdtype
     assert o.dtype == dtype and o.shape == (B, H, Nq, D) and lse.shape == (B, H, Nq)
     assert_close("O", o.cpu(), o_ref, scaled=True)
     assert max_abs(lse.cpu(), lse_ref) < LSE_TOL
+
+
+BWD_CASES = [
+    # B, H, Nq, Nk, D, config, scale dtype
+    (1, 2, 16, 32, 128, "normal", torch.float16),
+    (1, 2, 16, 160, 128, "normal", torch.float16),       # tiles on every wave, a second one on wave 0
+    (2, 3, 16, 3000, 128, "normal", torch.float16),      # reference benchmark shape (compute_flops.py:96)
+    (2, 3, 16, 3000, 64, "offset", torch.float16),
+    (1, 2, 1, 1, 128, "normal", torch.float16),
+    (1, 2, 5, 33, 64, "uniform", torch.float32),
+    (2, 2, 32, 689, 128, "offset", torch.float32),
+    (1, 2, 17, 1023, 128, "outlier", torch.float16),
+    (1, 4, 32, 512, 64, "normal", torch.float16),
+]
+
+
+@pytest.mark.parametrize("B,H,Nq,Nk,D,config,sdtype", BWD_CASES)
+def test_shared_kv_backward_vs_oracle(qfa, B, H, Nq, Nk, D, config, sdtype):
+    """dQ and dKV = dV + dK (quant_flash_attn.py:153-161) against fp64 autograd-checked formulas on
+    the dequantized tensor; bound 2e-2 * max(1, max|reference|) and cosine >= 0.999."""
+    q, kv = _inputs(config, B, H, Nq, Nk, D, torch.float16, seed=Nq + Nk + D)
+    g = torch.Generator().manual_seed(Nk)
+    do = torch.randn((B, H, Nq, D), generator=g).to(torch.float16)
+    sm = 1.0 / math.sqrt(D)
+    codes, scale, zp = qfa.asymmetric_quant_per_token(kv.to(DEV), scale_dtype=sdtype)
+    o, lse = qfa.attn_fwd_shared_kv(q.to(DEV), codes, scale, zp, sm)
+    dq, dkv = qfa.attn_bwd_shared_kv(q.to(DEV), codes, scale, zp, o, do.to(DEV), lse, sm)
+    torch.cuda.synchronize()
+    dq_ref, dkv_ref = oracle.legacy_bwd(q, codes.cpu(), scale.cpu(), zp.cpu(), do, sm)
+    assert dq.shape == (B, H, Nq, D) and dkv.shape == (B, H, Nk, D) and dq.dtype == torch.float16
+    # with a single key P = 1 and dS = 0: dQ is exactly zero and its cosine undefined
+    assert_close("dQ", dq.cpu(), dq_ref, scaled=True, cos_tol=COS_TOL if Nk > 1 else -1.0)
+    assert_close("dKV", dkv.cpu(), dkv_ref, scaled=True)
+
+
+def test_shared_kv_entry_point_autograd(qfa):
+    """The reference's entry point end to end on its benchmark shape (small batch): forward and
+    backward run the shared-KV kernels and kv_fp16 receives dKV (quant_flash_attn.py:178-237)."""
+    B, H, Nq, Nk, D = 2, 4, 16, 3000, 128
+    q, kv = _inputs("normal", B, H, Nq, Nk, D, torch.float16, seed=11)
+    sm = 1.0 / math.sqrt(D)
+    qd = q.to(DEV).requires_grad_(True)
+    kvd = kv.to(DEV).requires_grad_(True)
+    kv_quant = qfa.asymmetric_quant_per_token(kvd.detach())
+    o = qfa.quant_flash_attn(qd, kvd, kv_quant, sm)
+    do = torch.randn(o.shape, generator=torch.Generator().manual_seed(3)).to(torch.float16)
+    o.backward(do.to(DEV))
+    codes, scale, zp = (t.cpu() for t in kv_quant)
+    o_ref, _ = oracle.legacy_fwd(q, codes, scale, zp, sm)
+    dq_ref, dkv_ref = oracle.legacy_bwd(q, codes, scale, zp, do, sm)
+    assert_close("O", o.detach().cpu(), o_ref, scaled=True)
+    assert_close("dQ", qd.grad.cpu(), dq_ref, scaled=True)
+    assert_close("dKV", kvd.grad.cpu(), dkv_ref, scaled=True)
+    assert kvd.grad.dtype == torch.float16 and qd.grad.dtype == torch.float16
 
 
 def test_shared_kv_offsets_cancel(qfa):
