@@ -46,7 +46,8 @@ constexpr int SKVB_NBUF = 2;   // LDS slots per wave: the tile in work and the n
 template <int D> struct SkvBwdSmem {
   static constexpr int K_BYTES = SKV_TILE * D;
   static constexpr int SLOT = K_BYTES + 2 * SKV_TILE * 4;   // codes, one dword per key for scale and zero point
-  static constexpr int XT = 32 * 64;                        // (ds * scale) as binary16 [key][query]
+  static constexpr int XT = 32 * 128;                       // (ds * scale) as binary16 [key][query] (first half); later
+                                                            // 64 columns of the tile's dKV rows on their way out
   static constexpr int WAVE = SKVB_NBUF * SLOT + XT;
   static constexpr int ROWS = 32 * D * 2;                   // Q, then dO: binary16 [32][D], chunks swizzled
   static constexpr int OFF_Q = 4 * WAVE;
@@ -57,6 +58,13 @@ template <int D> struct SkvBwdSmem {
   static_assert(3 * MG * 4 <= OFF_STAT, "the dQ merge area overlays the slots and the Q / dO rows");
   static_assert(OFF_Q % 256 == 0, "row offsets are XOR-ed with block offsets");
 };
+
+// Chunk swizzle of the binary16 Q / dO rows (CPR 16-byte chunks each): distinct for 8 (16) consecutive
+// rows read at one chunk index, and moving whole 32-byte pairs apart for 4 consecutive rows, which is
+// what the transposing reads touch together.
+template <int CPR> __device__ __forceinline__ int row_swizzle(int i) {
+  return (2 * (i % 4) + (i / 4) % 2 + 8 * ((i / 8) % 2)) % CPR;
+}
 
 template <int OFF> __device__ __forceinline__ u32x2 lds_tr16(unsigned addr) { return lds_read_tr16_async<OFF>(addr); }
 
@@ -134,7 +142,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_bwd_k
         rd += d0 + d1;
         dsum += lo_to_f32<_Float16>(ov[e]) * d0 + hi_to_f32<_Float16>(ov[e]) * d1;
       }
-      const int off = pi * (D * 2) + ((c ^ (pi % CPR)) << 4);
+      const int off = pi * (D * 2) + ((c ^ row_swizzle<CPR>(pi)) << 4);
       *reinterpret_cast<u32x4 *>(smem + SM::OFF_Q + off) = qv;
       *reinterpret_cast<u32x4 *>(smem + SM::OFF_DO + off) = dv;
     }
@@ -172,7 +180,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_bwd_k
   // ---- per-lane LDS offsets
   const unsigned lds0 = lds_addr(smem);
   // (a) rows of Q / dO as A operands: row lr, chunk 4jj + 2g + hf for k-step 2jj + hf
-  const int row_off = lr * (D * 2), row_swz = lr % CPR;
+  const int row_off = lr * (D * 2), row_swz = row_swizzle<CPR>(lr);
   // (b) code rows as B operands: row lr, chunk 2jj + g (16 bytes = two k-steps)
   const int k_off = lr * D, k_swz = KSW::swz(lr);
   const int s16 = lane % 16, G = lane / 16;
@@ -186,7 +194,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_bwd_k
     for (int r = 0; r < 2; ++r) {
       const int i = 16 * hh + 8 * r + 4 * g + s16 / 4;
       const int chunk = 2 * (G % 2) + (s16 % 4) / 2;
-      qt_off[hh][r] = lds0 + SM::OFF_Q + i * (D * 2) + ((chunk ^ (i % CPR)) << 4) + 8 * (s16 % 2);
+      qt_off[hh][r] = lds0 + SM::OFF_Q + i * (D * 2) + ((chunk ^ row_swizzle<CPR>(i)) << 4) + 8 * (s16 % 2);
     }
   // (d) ds*scale: written as [key lr][query], 8-byte segment seg = 2aa + g at position seg ^ ((key/2) % 8);
   //     read back transposed: lane s addresses key 16kk + 8g + 4r + s/4, segment 4(G%2) + s%4
@@ -310,8 +318,11 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_bwd_k
   auto tile_dkv = [&](int i) {
     // ---- 4. dKV^T = dO^T P + Q^T dS for one block of 32 d at a time; column = this lane's key
     const int j0 = (wave + 4 * i) * SKV_TILE;
-    const bool key_ok = j0 + lr < a.Nk;
-    _Float16 *krow = dkv_bh + (int64_t)(j0 + lr) * a.sdkn;
+    unsigned char *stage = smem + wave_off + SKVB_NBUF * SM::SLOT;
+    // two blocks (64 columns, 128 bytes a row) are staged in LDS and leave as whole 128-byte lines:
+    // 16-byte pair p of row j sits at position p ^ (j % 8)
+    const int st_w = lr * 128 + 8 * g, st_wswz = lr % 8;
+    const int st_r = (lane / 8) * 128 + (((lane % 8) ^ (lane / 8)) << 4);
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
       u32x2 fr[2][2][2];   // [matrix: dO, Q][hh][r]
@@ -333,13 +344,19 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_bwd_k
         acc = mfma_h(u32x4{d0[0], d0[1], d1[0], d1[1]}, pf[hh], acc);
         acc = mfma_h(u32x4{q0[0], q0[1], q1[0], q1[1]}, df[hh], acc);
       }
-      if (key_ok) {
 #pragma unroll
-        for (int aa = 0; aa < 4; ++aa) {
-          u32x2 o2;
-          o2[0] = pack_h2(acc[4 * aa], acc[4 * aa + 1]);
-          o2[1] = pack_h2(acc[4 * aa + 2], acc[4 * aa + 3]);
-          *reinterpret_cast<u32x2 *>(krow + 32 * db + 8 * aa + 4 * g) = o2;
+      for (int aa = 0; aa < 4; ++aa) {
+        u32x2 o2;
+        o2[0] = pack_h2(acc[4 * aa], acc[4 * aa + 1]);
+        o2[1] = pack_h2(acc[4 * aa + 2], acc[4 * aa + 3]);
+        *reinterpret_cast<u32x2 *>(stage + st_w + (((4 * (db % 2) + aa) ^ st_wswz) << 4)) = o2;
+      }
+      if (db % 2 == 1) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const u32x4 row16 = *reinterpret_cast<const u32x4 *>(stage + st_r + it * 1024);
+          const int j = j0 + 8 * it + lane / 8;
+          if (j < a.Nk) *reinterpret_cast<u32x4 *>(dkv_bh + (int64_t)j * a.sdkn + 32 * (db - 1) + 8 * (lane % 8)) = row16;
         }
       }
     }
