@@ -176,6 +176,31 @@ def main():
     extra["qk_stage_int8_tops"] = round(0.5 * F_fwd / (ms_qk * 1e-3) / 1e12, 2)
     extra["qk_stage_frac_int8_peak"] = round(0.5 * F_fwd / (ms_qk * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)
 
+    # ---- the reference's own benchmark shape (compute_flops.py:96): shared K = V codes, fp16 Q, 16 queries
+    # against 3000 keys.  HBM-bound: bytes = calculate_theoretical_io of compute_flops.py:39-83.
+    def shared_kv_leg(D2):
+        Z2, H2, Nq2, Nk2 = 512, 16, 16, 3000
+        g2 = torch.Generator(device=dev).manual_seed(1)
+        kv2 = torch.randn((Z2, H2, Nk2, D2), generator=g2, device=dev, dtype=torch.float16)
+        codes2, scale2, zp2 = qfa.asymmetric_quant_per_token(kv2)
+        del kv2
+        q2 = torch.randn((Z2, H2, Nq2, D2), generator=g2, device=dev, dtype=torch.float16)
+        do2 = torch.randn((Z2, H2, Nq2, D2), generator=g2, device=dev, dtype=torch.float16)
+        sm2 = 1.0 / math.sqrt(D2)
+        o2, lse2 = qfa.attn_fwd_shared_kv(q2, codes2, scale2, zp2, sm2)
+        mf = time_events(lambda: qfa.attn_fwd_shared_kv(q2, codes2, scale2, zp2, sm2), 20, 5)
+        mb = time_events(lambda: qfa.attn_bwd_shared_kv(q2, codes2, scale2, zp2, o2, do2, lse2, sm2), 10, 3)
+        io_f = Z2 * H2 * (Nq2 * D2 * 2 * 2 + Nq2 * 4 + Nk2 * (D2 + 3))
+        io_b = Z2 * H2 * (4 * Nq2 * D2 * 2 + 2 * Nq2 * 4 + Nk2 * (D2 + 3) + Nk2 * D2 * 2)
+        fl = 4.0 * Z2 * H2 * Nq2 * Nk2 * D2
+        return {"fwd_ms": round(mf, 4), "fwd_GBps": round(io_f / mf / 1e6, 1),
+                "fwd_frac_hbm_peak": round(io_f / mf / 1e6 / PEAK_HBM_GBS, 4), "fwd_tflops": round(fl / mf / 1e9, 2),
+                "bwd_ms": round(mb, 4), "bwd_GBps": round(io_b / mb / 1e6, 1),
+                "bwd_frac_hbm_peak": round(io_b / mb / 1e6 / PEAK_HBM_GBS, 4), "bwd_tflops": round(2.5 * fl / mb / 1e9, 2)}
+    extra["shared_kv_Z512_H16_Nq16_Nkv3000_D128_fp16"] = shared_kv_leg(128)
+    if args.all_configs:
+        extra["shared_kv_Z512_H16_Nq16_Nkv3000_D64_fp16"] = shared_kv_leg(64)
+
     if args.sdpa:
         import torch.nn.functional as Fn
         qs, ks, vs = (t.clone().requires_grad_(True) for t in (q, k, v))
