@@ -11,6 +11,11 @@ are derived here, once, from sources independent of the code they check:
                    O / LSE / dQ / dK / dV evaluated in fp64 by plain torch formulas written out below
                    (softmax(sm * Q^ K^^T + mask) V and torch.autograd), independent of oracle.attn_*.
 
+  shared_kv_small.npz  two small problems of the reference's own operator (quant_flash_attn.py:22-166: one
+                   quantized tensor is K and V, Q stays fp16): q / kv / dO as fp16 bit patterns, the exactly
+                   quantized kv (codes, fp16 scale as stored by the reference, zero point), and O / LSE /
+                   dQ / dKV from plain fp64 torch formulas + autograd on kv^ = (codes - zp) * fp16(scale).
+
 Fixtures are data only; the tests that read them are tests/test_golden.py (CPU: oracle vs fixtures;
 GPU: kernels vs fixtures)."""
 import json
@@ -90,6 +95,29 @@ def attn_case(seed, B, H, Nq, Nk, D, causal, quantize):
             "causal": np.array(int(causal)), "sm_scale": np.array(sm, dtype=np.float64)}
 
 
+def f16_bits(t: torch.Tensor) -> np.ndarray:
+    return t.to(torch.float16).view(torch.int16).numpy().view(np.uint16)
+
+
+def shared_kv_case(seed, B, H, Nq, Nk, D, quantize):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, H, Nq, D, generator=g).to(torch.float16)
+    kv = (torch.randn(B, H, Nk, D, generator=g) + 0.5 * torch.randn(B, H, Nk, 1, generator=g)).to(torch.float16)
+    do = torch.randn(B, H, Nq, D, generator=g).to(torch.float16)
+    sm = 1.0 / math.sqrt(D)
+    codes, zp, scale32 = quantize(kv)
+    scale16 = scale32.to(torch.float16)                     # what the reference stores (asymmetric_quant.py:93,128)
+    kvh = ((codes.double() - zp.double()[..., None]) * scale16.double()[..., None]).requires_grad_(True)
+    qd = q.double().requires_grad_(True)
+    s = sm * qd @ kvh.transpose(-1, -2)
+    lse = torch.logsumexp(s, dim=-1)
+    o = torch.softmax(s, dim=-1) @ kvh
+    o.backward(do.double())
+    return {"q": f16_bits(q), "kv": f16_bits(kv), "do": f16_bits(do), "codes": codes.numpy(), "zp": zp.numpy(),
+            "scale16": f16_bits(scale16), "o": o.detach().float().numpy(), "lse": lse.detach().float().numpy(),
+            "dq": qd.grad.float().numpy(), "dkv": kvh.grad.float().numpy(), "sm_scale": np.array(sm, dtype=np.float64)}
+
+
 def quantize_exact(x: torch.Tensor):
     """Quantize every row with the exact-rational model (slow, small inputs only)."""
     xs = x.to(torch.float32)
@@ -114,4 +142,8 @@ if __name__ == "__main__":
              "ragged_Nq24_Nk72_D128": attn_case(8, 1, 1, 24, 72, 128, False, quantize_exact)}
     flat = {f"{name}/{key}": val for name, c in cases.items() for key, val in c.items()}
     np.savez_compressed(os.path.join(HERE, "attn_small.npz"), **flat)
+    skv = {"Nq16_Nk100_D128": shared_kv_case(9, 1, 2, 16, 100, 128, quantize_exact),
+           "Nq5_Nk70_D64": shared_kv_case(10, 1, 1, 5, 70, 64, quantize_exact)}
+    np.savez_compressed(os.path.join(HERE, "shared_kv_small.npz"),
+                        **{f"{name}/{key}": val for name, c in skv.items() for key, val in c.items()})
     print("wrote", os.listdir(HERE))

@@ -107,3 +107,53 @@ def test_kernels_meet_attention_known_answers(qfa):
         assert_close(f"{name} dQ", dq.cpu(), torch.from_numpy(c["dq"]).double(), scaled=True)
         assert_close(f"{name} dK", dk.cpu(), torch.from_numpy(c["dk"]).double(), scaled=True)
         assert_close(f"{name} dV", dv.cpu(), torch.from_numpy(c["dv"]).double(), scaled=True)
+
+
+def _shared_kv_cases():
+    z = np.load(os.path.join(GOLDEN, "shared_kv_small.npz"), allow_pickle=False)
+    names = sorted({k.split("/")[0] for k in z.files})
+    return {n: {k.split("/")[1]: z[k] for k in z.files if k.startswith(n + "/")} for n in names}
+
+
+def _f16(bits: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(bits.view(np.int16).copy()).view(torch.float16)
+
+
+def test_oracle_shared_kv_reproduces_known_answers():
+    """oracle.legacy_fwd / legacy_bwd (quant_flash_attn.py:22-166 restated) against the fixture's plain
+    fp64 formulas, and the oracle quantizer against the fixture's exactly quantized kv."""
+    cases = _shared_kv_cases()
+    assert set(cases) == {"Nq16_Nk100_D128", "Nq5_Nk70_D64"}
+    for name, c in cases.items():
+        q, kv, do = _f16(c["q"]), _f16(c["kv"]), _f16(c["do"])
+        codes, scale16, zp, _, _ = oracle.quantize_per_token(kv, torch.float16)
+        assert np.array_equal(codes.numpy(), c["codes"]), name
+        assert np.array_equal(zp.reshape(c["zp"].shape).numpy(), c["zp"]), name
+        assert torch.equal(scale16.reshape(c["scale16"].shape), _f16(c["scale16"])), name
+        sm = float(c["sm_scale"])
+        o, lse = oracle.legacy_fwd(q, codes, scale16, zp, sm)
+        dq, dkv = oracle.legacy_bwd(q, codes, scale16, zp, do, sm)
+        for got, key in ((o, "o"), (lse, "lse"), (dq, "dq"), (dkv, "dkv")):
+            ref = torch.from_numpy(c[key]).double()
+            assert (got.double().reshape(ref.shape) - ref).abs().max() <= 2e-6 * max(1.0, ref.abs().max().item()), (name, key)
+
+
+@pytest.mark.gpu
+def test_kernels_meet_shared_kv_known_answers(qfa):
+    """The reference's entry point end to end (quantizer + shared-KV forward + backward kernels)."""
+    for name, c in _shared_kv_cases().items():
+        q = _f16(c["q"]).to(DEV).requires_grad_(True)
+        kv = _f16(c["kv"]).to(DEV).requires_grad_(True)
+        sm = float(c["sm_scale"])
+        kv_quant = qfa.asymmetric_quant_per_token(kv.detach())
+        assert np.array_equal(kv_quant[0].cpu().numpy(), c["codes"]), name
+        assert np.array_equal(kv_quant[2].cpu().reshape(c["zp"].shape).numpy(), c["zp"]), name
+        assert torch.equal(kv_quant[1].cpu().reshape(c["scale16"].shape), _f16(c["scale16"])), name
+        o = qfa.quant_flash_attn(q, kv, kv_quant, sm)
+        o.backward(_f16(c["do"]).to(DEV))
+        _, lse = qfa.attn_fwd_shared_kv(q.detach(), *kv_quant, sm)
+        torch.cuda.synchronize()
+        assert_close(f"{name} O", o.detach().cpu(), torch.from_numpy(c["o"]).double(), scaled=True)
+        assert (lse.cpu().double().reshape(c["lse"].shape) - torch.from_numpy(c["lse"]).double()).abs().max() < 2.0 ** -8
+        assert_close(f"{name} dQ", q.grad.cpu(), torch.from_numpy(c["dq"]).double(), scaled=True)
+        assert_close(f"{name} dKV", kv.grad.cpu(), torch.from_numpy(c["dkv"]).double(), scaled=True)
