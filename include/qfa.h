@@ -114,13 +114,15 @@ int qfa_attn_fwd_shared_kv(const void *q, const int8_t *codes, const void *scale
                            int64_t soh, int64_t son, float sm_scale, void *stream);
 
 /*
- * Backward of qfa_attn_fwd_shared_kv for one short query block (Nq <= 32), fp16:
+ * Backward of qfa_attn_fwd_shared_kv, fp16:
  *     P = exp(sm_scale Q KV^T - LSE),  dP = dO KV^T,  dS = sm_scale P o (dP - delta),  delta = rowsum(O o dO)
  *     dQ = dS KV,    dKV = P^T dO + dS^T Q
  * Replaces the launches made by QuantFlashAttention.backward (quant_flash_attn.py:207-237):
  * _bwd_preprocess_kernel (:87-101; delta is computed inside) and _attn_bwd_kernel_quantized
- * (:104-166), which also stores the single gradient dKV = dV + dK (:161).  One workgroup per
- * (batch, head) streams the codes once and writes each dKV row once.
+ * (:104-166), which also stores the single gradient dKV = dV + dK (:161).  Up to 32 queries per
+ * (batch, head) run in one fused pass (one workgroup per (batch, head) streams the codes once and
+ * writes each dKV row once); longer query blocks run a dQ kernel (one workgroup per 16 queries) and
+ * a dKV kernel (one workgroup per 128 keys walking over the queries).
  *   q, o, dout, dq [B,H,Nq,D] and dkv [B,H,Nk,D] fp16 (io_dtype must be QFA_F16), strides as given;
  *   codes, scale, scale_dtype, zp, lse as in the forward.  D in {64, 128}.
  *   The sums of a query's and of a dO row's D elements must stay inside binary16 range.

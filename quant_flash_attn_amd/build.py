@@ -22,7 +22,7 @@ COMMON = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # the quantizer must evaluate its expressions as single IEEE operations (bit-exact codes)
 PER_FILE = {"qfa_quant.hip": ["-ffp-contract=off", "-fno-fast-math"]}
-SOURCES = ["qfa_api.cpp", "qfa_quant.hip", "qfa_fwd.hip", "qfa_bwd.hip", "qfa_skv.hip", "qfa_skv_bwd.hip"]
+SOURCES = ["qfa_api.cpp", "qfa_quant.hip", "qfa_fwd.hip", "qfa_bwd.hip", "qfa_skv.hip", "qfa_skv_bwd.hip", "qfa_skv_bwd_long.hip"]
 
 
 def _hipcc() -> str:

@@ -173,12 +173,11 @@ int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale
   if (int e = check_shared_kv(who, a)) return e;
   if (!dout || !dq || !dkv) return set_error(QFA_EINVAL, "%s: null pointer argument", who);
   if (io_dtype != QFA_F16) return set_error(QFA_EUNSUPPORTED, "%s: io_dtype must be QFA_F16", who);
-  if (Nq > 32) return set_error(QFA_EUNSUPPORTED, "%s: at most 32 queries per (batch, head), got %lld", who, (long long)Nq);
   if (!aligned16(dout) || !aligned16(dq) || !aligned16(dkv))
     return set_error(QFA_EINVAL, "%s: dout, dq, dkv must be 16-byte aligned", who);
   if (!strides_ok(sdob, sdoh, sdon, D, 2) || !strides_ok(sdqb, sdqh, sdqn, D, 2) || !strides_ok(sdkb, sdkh, sdkn, D, 2))
     return set_error(QFA_EINVAL, "%s: strides must be positive multiples of 16 bytes, token stride >= D", who);
-  return launch_skv_bwd(a, (hipStream_t)stream);
+  return Nq <= 32 ? launch_skv_bwd(a, (hipStream_t)stream) : launch_skv_bwd_long(a, (hipStream_t)stream);
 }
 
 int qfa_bench_qk_stage(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,

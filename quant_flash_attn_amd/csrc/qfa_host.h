@@ -53,6 +53,7 @@ struct SkvAttnArgs {
   int D, io_dtype, scale_dtype;
 };
 int launch_skv_fwd(const SkvAttnArgs &a, hipStream_t st);
-int launch_skv_bwd(const SkvAttnArgs &a, hipStream_t st);   // io_dtype QFA_F16, Nq <= 32
+int launch_skv_bwd(const SkvAttnArgs &a, hipStream_t st);        // io_dtype QFA_F16, Nq <= 32: one fused pass
+int launch_skv_bwd_long(const SkvAttnArgs &a, hipStream_t st);   // io_dtype QFA_F16, any Nq: dQ kernel + dKV kernel
 
 }  // namespace qfa

@@ -42,20 +42,6 @@ struct SkvArgs {
   int BH;        // batch * heads
 };
 
-// The kernel works on blocks of 16 queries (the reference's benchmark shape has exactly 16) with the
-// 16x16x32 MFMA: a 32-key tile is two 16-key row blocks of S^T and one k-step of O^T.  A lane owns
-// query lane%16 and the keys 16rb + 4(lane/16) + {0..3} of each tile.
-__device__ __forceinline__ f32x4 mfma_h16(u32x4 a, u32x4 b, f32x4 c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-}
-// Chunk swizzle of a code tile for this kernel: as Swz<D>, plus a term in row/16 so that the eight keys
-// one transposing read touches (4G + {0..3} and 16 + 4G + {0..3}) fall into different bank groups.
-template <int D> struct SwzSkv {
-  static constexpr int CPR = D / 16;
-  static __device__ __forceinline__ int swz(int row) {
-    return D == 128 ? ((row / 2) ^ ((row / 16) * 4)) % 8 : ((row / 4) ^ ((row / 16) * 2)) % 4;
-  }
-};
 constexpr int SKV_NBUF = 3;
 
 template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) void skv_fwd_kernel(SkvArgs a) {

@@ -40,6 +40,45 @@ __device__ __forceinline__ u32x2 lds_read_tr8_async(unsigned addr) {
   return r;
 }
 
+// 16x16x32 MFMA, used on blocks of 16 queries: a 32-key tile is two 16-key row blocks of S^T and one
+// k-step of the products contracted over keys.  A lane owns query lane%16 and the keys
+// 16rb + 4(lane/16) + {0..3} of each tile.
+__device__ __forceinline__ f32x4 mfma_h16(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+// Chunk swizzle of a code tile for the 16-query kernels: as Swz<D>, plus a term in row/16 so that the eight
+// keys one transposing read touches (4G + {0..3} and 16 + 4G + {0..3}) fall into different bank groups.
+template <int D> struct SwzSkv {
+  static constexpr int CPR = D / 16;
+  static __device__ __forceinline__ int swz(int row) {
+    return D == 128 ? ((row / 2) ^ ((row / 16) * 4)) % 8 : ((row / 4) ^ ((row / 16) * 2)) % 4;
+  }
+};
+
+// Copy of 32-key tile t of one (batch, head) into an LDS slot by direct global->LDS loads: the codes
+// through `cp` (rows dense, chunks swizzled), then one dword per key for the scale and one for the zero
+// point (sub-dword direct loads write lane l's zero-extended value to the dword at 4*l).  Rows past the
+// end of the sequence read as zeros.  Copy::N + 2 vector-memory instructions per wave.
+template <typename S, int D, typename Copy>
+__device__ __forceinline__ void skv_issue_tile(const Copy &cp, unsigned char *slot, const unsigned char *codes_bh,
+                                               const void *scale, const int8_t *zp, int64_t tk0, int t, int Nk,
+                                               int64_t scn, int lane) {
+  const int rows = min(SKV_TILE, Nk - t * SKV_TILE);
+  const rsrc_t rs_k = make_rsrc(codes_bh + (int64_t)t * SKV_TILE * scn, (unsigned)((rows - 1) * (int)scn + D));
+#pragma unroll
+  for (int c = 0; c < Copy::N; ++c) cp.issue_one(rs_k, slot, 0, lane, c);
+  const rsrc_t rs_s = make_rsrc(reinterpret_cast<const S *>(scale) + tk0 + (int64_t)t * SKV_TILE,
+                                (unsigned)rows * (unsigned)sizeof(S));
+  const rsrc_t rs_z = make_rsrc(zp + tk0 + (int64_t)t * SKV_TILE, (unsigned)rows);
+  if (lane < SKV_TILE) {
+    if constexpr (sizeof(S) == 4)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_s, (lptr_t)(slot + SKV_TILE * D), 4, lane * 4, 0, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_s, (lptr_t)(slot + SKV_TILE * D), 2, lane * 2, 0, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_z, (lptr_t)(slot + SKV_TILE * D + SKV_TILE * 4), 1, lane, 0, 0, 0);
+  }
+}
+
 // wait for every LDS operation of this wave; `tie` keeps the users of an asynchronously loaded
 // register pair behind the wait that precedes it in program order
 __device__ __forceinline__ void lds_wait_all() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }

@@ -11,9 +11,8 @@ Two autograd entry points, both backed by the HIP kernels behind qfa_attn_fwd / 
       The reference's own entry point (quant_flash_attn.py:173-240): one quantized tensor serves as
       K and V, `kv_fp16` only receives the gradient, backward returns (dq, dkv, None, None) with
       dkv = dK + dV (:161).  Query blocks of up to SHARED_KV_MAX_Q tokens run the reference's
-      computation itself in the forward (Q in 16-bit, qfa_attn_fwd_shared_kv), and fp16 blocks of
-      up to SHARED_KV_BWD_MAX_Q tokens also in the backward (qfa_attn_bwd_shared_kv).  Everything
-      else goes through the INT8-score kernels, where Q is quantized per token too (stated
+      computation itself in the forward (Q in 16-bit, qfa_attn_fwd_shared_kv), and in fp16 also in
+      the backward (qfa_attn_bwd_shared_kv).  Everything else goes through the INT8-score kernels, where Q is quantized per token too (stated
       difference from the reference, which keeps Q in fp16).
 """
 from __future__ import annotations
@@ -157,16 +156,13 @@ def attn_fwd_shared_kv(q: torch.Tensor, codes: torch.Tensor, scale: torch.Tensor
     return o, lse
 
 
-# Largest query block of the shared-KV backward kernel (one 32-row MFMA block of queries).
-SHARED_KV_BWD_MAX_Q = 32
-
-
 def attn_bwd_shared_kv(q: torch.Tensor, codes: torch.Tensor, scale: torch.Tensor, zero_point: torch.Tensor,
                        o: torch.Tensor, do: torch.Tensor, lse: torch.Tensor, sm_scale: float
                        ) -> Tuple[torch.Tensor, torch.Tensor]:
     """dQ, dKV of attn_fwd_shared_kv in fp16: the computation of _attn_bwd_kernel_quantized
     (quant_flash_attn.py:104-166) with dKV = dV + dK as stored there (:161).  q, o, do fp16
-    [B,H,Nq,D] with Nq <= 32; lse as returned by the forward."""
+    [B,H,Nq,D]; lse as returned by the forward.  Up to 32 queries run in one fused pass over the codes,
+    longer blocks in a dQ kernel plus a dKV kernel."""
     if q.dtype != torch.float16 or o.dtype != torch.float16:
         raise TypeError("the shared-KV backward kernel computes in float16: q and o must be float16")
     if codes.dim() != 4 or codes.dtype != torch.int8:
@@ -267,7 +263,7 @@ class QuantFlashAttention(torch.autograd.Function):
         t = ctx.saved_tensors
         if ctx.shared_kv:
             q, codes, scale, zp, o, lse = t
-            if q.dtype == torch.float16 and q.shape[2] <= SHARED_KV_BWD_MAX_Q:
+            if q.dtype == torch.float16:
                 dq, dkv = attn_bwd_shared_kv(q, codes, scale, zp, o, grad_output, lse, ctx.sm_scale)
                 return dq, dkv.to(ctx.kv_dtype), None, None
             qq, kq, v16 = _legacy_operands(q, codes, scale, zp, q.dtype)

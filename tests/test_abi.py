@@ -74,7 +74,7 @@ def test_argument_errors_need_no_gpu(qfa):
         sq, sc = (Nq * D, Nq * D, D), (Nk * D, Nk * D, D)
         return L.qfa_attn_bwd_shared_kv(ok_ptr, ok_ptr, ok_ptr, 0, ok_ptr, ok_ptr, ok_ptr, ok_ptr, ok_ptr, dkv, io,
                                         1, 1, Nq, Nk, D, *sq, *sc, *sq, *sq, *sq, *sc, 0.1, None)
-    assert skv_bwd(Nq=33) == -2 and b"at most 32 queries" in L.qfa_last_error()
+    assert skv_bwd(D=96) == -2 and b"head_dim" in L.qfa_last_error()
     assert skv_bwd(io=2) == -2 and b"QFA_F16" in L.qfa_last_error()
     assert skv_bwd(dkv=None) == -1 and b"null" in L.qfa_last_error()
 

@@ -62,6 +62,11 @@ BWD_CASES = [
     (2, 2, 32, 689, 128, "offset", torch.float32),
     (1, 2, 17, 1023, 128, "outlier", torch.float16),
     (1, 4, 32, 512, 64, "normal", torch.float16),
+    # more than 32 queries: dQ kernel + dKV kernel
+    (2, 2, 97, 689, 128, "normal", torch.float16),       # reference test shape (test_accuracy.py:44), small batch
+    (1, 3, 33, 100, 64, "offset", torch.float32),        # one query past a block, one key chunk
+    (1, 2, 128, 1000, 128, "uniform", torch.float16),
+    (2, 2, 64, 129, 64, "outlier", torch.float32),       # second key chunk holds a single key
 ]
 
 
@@ -103,6 +108,26 @@ def test_shared_kv_entry_point_autograd(qfa):
     assert_close("dQ", qd.grad.cpu(), dq_ref, scaled=True)
     assert_close("dKV", kvd.grad.cpu(), dkv_ref, scaled=True)
     assert kvd.grad.dtype == torch.float16 and qd.grad.dtype == torch.float16
+
+
+def test_shared_kv_entry_point_long_query_block(qfa):
+    """97 queries (a reference test shape, test_accuracy.py:44): the forward splits them over workgroups
+    of 16, the backward runs its dQ and dKV kernels."""
+    B, H, Nq, Nk, D = 2, 3, 97, 689, 128
+    q, kv = _inputs("normal", B, H, Nq, Nk, D, torch.float16, seed=12)
+    sm = 1.0 / math.sqrt(D)
+    qd = q.to(DEV).requires_grad_(True)
+    kvd = kv.to(DEV).requires_grad_(True)
+    kv_quant = qfa.asymmetric_quant_per_token(kvd.detach())
+    o = qfa.quant_flash_attn(qd, kvd, kv_quant, sm)
+    do = torch.randn(o.shape, generator=torch.Generator().manual_seed(4)).to(torch.float16)
+    o.backward(do.to(DEV))
+    codes, scale, zp = (t.cpu() for t in kv_quant)
+    o_ref, _ = oracle.legacy_fwd(q, codes, scale, zp, sm)
+    dq_ref, dkv_ref = oracle.legacy_bwd(q, codes, scale, zp, do, sm)
+    assert_close("O", o.detach().cpu(), o_ref, scaled=True)
+    assert_close("dQ", qd.grad.cpu(), dq_ref, scaled=True)
+    assert_close("dKV", kvd.grad.cpu(), dkv_ref, scaled=True)
 
 
 def test_shared_kv_offsets_cancel(qfa):
