@@ -10,7 +10,7 @@ Two autograd entry points, both backed by the HIP kernels behind qfa_attn_fwd / 
   QuantFlashAttention.apply(q, kv_fp16, kv_quant, sm_scale)     (alias quant_flash_attn)
       The reference's own entry point (quant_flash_attn.py:173-240): one quantized tensor serves as
       K and V, `kv_fp16` only receives the gradient, backward returns (dq, dkv, None, None) with
-      dkv = dK + dV (:161).  Query blocks of up to SHARED_KV_MAX_Q tokens run the reference's
+      dkv = dK + dV (:161).  Query blocks of up to SHARED_KV_MAX_Q (512) tokens run the reference's
       computation itself in the forward (Q in 16-bit, qfa_attn_fwd_shared_kv), and in fp16 also in
       the backward (qfa_attn_bwd_shared_kv).  Everything else goes through the INT8-score kernels, where Q is quantized per token too (stated
       difference from the reference, which keeps Q in fp16).
@@ -119,9 +119,11 @@ def attn_bwd_quantized(qq: QuantizedTokens, kq: QuantizedTokens, v: torch.Tensor
     return dq, dk, dv
 
 
-# Longest query block the shared-KV kernel is used for: it re-reads the codes once per 32 queries,
-# which pays while the operator is bound by streaming them (the reference's decode-like shapes).
-SHARED_KV_MAX_Q = 128
+# Longest query block the shared-KV kernels are used for.  They stream the codes once per 16 queries
+# (from L2 after the first block), which wins while Nq is small against Nk -- the reference's test and
+# benchmark shapes; measured crossover with the INT8-score kernels at Nk=4096, D=128: between 512 and
+# 1024 queries (fwd 1.16 vs 1.51 ms at 512, 1.14 vs 1.01 ms at 1024).
+SHARED_KV_MAX_Q = 512
 
 
 def attn_fwd_shared_kv(q: torch.Tensor, codes: torch.Tensor, scale: torch.Tensor, zero_point: torch.Tensor,

@@ -121,7 +121,8 @@ def test_autograd_entry_points(qfa):
 
 
 @pytest.mark.parametrize("Z,H,Nq,Nkv,D", [(2, 4, 18, 512, 64), (2, 8, 32, 1024, 128), (4, 16, 16, 2048, 64), (1, 2, 17, 1023, 128),
-                                          (3, 5, 97, 689, 128)])
+                                          (3, 5, 97, 689, 128),      # the reference's shapes (test_accuracy.py:35-45, small batch)
+                                          (1, 2, 600, 700, 128)])    # query block past the shared-KV kernels: INT8-score path
 def test_reference_entry_point_shared_kv(qfa, Z, H, Nq, Nkv, D):
     """The reference's own test (test_accuracy.py:47-133): fp16 q, kv ~ N(0,1), seed 20, quantize kv
     externally, forward + backward, against un-quantized fp16-input attention at its tolerances
@@ -143,13 +144,17 @@ def test_reference_entry_point_shared_kv(qfa, Z, H, Nq, Nkv, D):
     assert torch.allclose(out.detach().cpu().double(), ref.detach(), atol=1e-1, rtol=0)
     assert torch.allclose(qg.grad.cpu().double(), qr.grad, atol=1e-2, rtol=1e-2)
     assert torch.allclose(kvg.grad.cpu().double(), kvr.grad, atol=1e-2, rtol=2e-2)
-    # shared-KV oracle on the same codes, Q quantized as this build does
+    # shared-KV oracle on the same codes: Q as it is for the shared-KV kernels (the reference's
+    # computation), quantized per token where the INT8-score kernels take over
+    from quant_flash_attn_amd.quant_flash_attn import SHARED_KV_MAX_Q
     codes, scale, zp = (t.cpu() for t in kv_quant)
-    qc, _, zq, sq, _ = oracle.quantize_per_token(q)
-    qh = oracle.dequantize_per_token(qc, sq, zq, torch.float64)
+    qh = q
+    if Nq > SHARED_KV_MAX_Q:
+        qc, _, zq, sq, _ = oracle.quantize_per_token(q)
+        qh = oracle.dequantize_per_token(qc, sq, zq, torch.float64)
     o_ref, _ = oracle.legacy_fwd(qh, codes, scale, zp, sm)
     dq_ref, dkv_ref = oracle.legacy_bwd(qh, codes, scale, zp, do, sm)
-    assert_close("O", out.detach().cpu(), o_ref)
+    assert_close("O", out.detach().cpu(), o_ref, scaled=True)
     assert_close("dQ", qg.grad.cpu(), dq_ref, scaled=True)
     assert_close("dKV", kvg.grad.cpu(), dkv_ref, scaled=True)
 
