@@ -107,11 +107,19 @@ int qfa_attn_fwd(const int8_t *qc, const float *sq, const int8_t *zq, const int3
  *   scale  [B*H*Nk] of scale_dtype: QFA_F32, or the same 16-bit type as io_dtype
  *   D in {64, 128}.  q, codes, o 16-byte aligned, strides multiples of 16 bytes, scn < 2^23.
  *   The sum of a query's D elements must stay inside binary16 range (|sum| < 65504).
+ *   workspace  nullable.  With few (batch, head) pairs one workgroup per 16 queries leaves most of the
+ *              chip idle (the reference launches one program per (batch, head)); given a caller-owned
+ *              scratch of qfa_attn_fwd_shared_kv_workspace_bytes(...) bytes (16-byte aligned; the
+ *              function returns 0 when no split pays) the keys of a query block are split over several
+ *              workgroups and a second small kernel merges their partial (O, m, l).  NULL: never split.
  */
+int64_t qfa_attn_fwd_shared_kv_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D);
+
 int qfa_attn_fwd_shared_kv(const void *q, const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp,
                            void *o, float *lse, int io_dtype, int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D,
                            int64_t sqb, int64_t sqh, int64_t sqn, int64_t scb, int64_t sch, int64_t scn, int64_t sob,
-                           int64_t soh, int64_t son, float sm_scale, void *stream);
+                           int64_t soh, int64_t son, float sm_scale, void *workspace, int64_t workspace_bytes,
+                           void *stream);
 
 /*
  * Backward of qfa_attn_fwd_shared_kv, fp16:

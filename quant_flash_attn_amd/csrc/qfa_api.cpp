@@ -140,10 +140,16 @@ static int check_shared_kv(const char *who, const SkvAttnArgs &a) {
   return 0;
 }
 
+int64_t qfa_attn_fwd_shared_kv_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D) {
+  if (B <= 0 || H <= 0 || Nq <= 0 || Nk <= 0 || (D != 64 && D != 128)) return 0;
+  return skv_fwd_workspace_bytes(B, H, Nq, Nk, D);
+}
+
 int qfa_attn_fwd_shared_kv(const void *q, const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp,
                            void *o, float *lse, int io_dtype, int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D,
                            int64_t sqb, int64_t sqh, int64_t sqn, int64_t scb, int64_t sch, int64_t scn, int64_t sob,
-                           int64_t soh, int64_t son, float sm_scale, void *stream) {
+                           int64_t soh, int64_t son, float sm_scale, void *workspace, int64_t workspace_bytes,
+                           void *stream) {
   SkvAttnArgs a;
   memset(&a, 0, sizeof(a));
   a.q = q; a.codes = codes; a.scale = scale; a.zp = zp; a.o = o; a.lse = lse;
@@ -151,6 +157,13 @@ int qfa_attn_fwd_shared_kv(const void *q, const int8_t *codes, const void *scale
   a.sqb = sqb; a.sqh = sqh; a.sqn = sqn; a.scb = scb; a.sch = sch; a.scn = scn; a.sob = sob; a.soh = soh; a.son = son;
   a.sm_scale = sm_scale;
   if (int e = check_shared_kv("attn_fwd_shared_kv", a)) return e;
+  if (workspace) {
+    const int64_t need = skv_fwd_workspace_bytes(B, H, Nq, Nk, D);
+    if (!aligned16(workspace) || workspace_bytes < need)
+      return set_error(QFA_EINVAL, "attn_fwd_shared_kv: workspace must be 16-byte aligned and hold %lld bytes "
+                       "(qfa_attn_fwd_shared_kv_workspace_bytes), got %lld", (long long)need, (long long)workspace_bytes);
+    a.workspace = need > 0 ? workspace : nullptr;
+  }
   return launch_skv_fwd(a, (hipStream_t)stream);
 }
 

@@ -46,6 +46,7 @@ struct SkvAttnArgs {
   const void *q; const int8_t *codes; const void *scale; const int8_t *zp;
   void *o; float *lse;
   const void *dout; void *dq; void *dkv;   // backward only
+  void *workspace;                         // forward only, nullable: partial results when the keys are split
   int64_t B, H, Nq, Nk;
   int64_t sqb, sqh, sqn, scb, sch, scn, sob, soh, son;
   int64_t sdob, sdoh, sdon, sdqb, sdqh, sdqn, sdkb, sdkh, sdkn;
@@ -53,6 +54,7 @@ struct SkvAttnArgs {
   int D, io_dtype, scale_dtype;
 };
 int launch_skv_fwd(const SkvAttnArgs &a, hipStream_t st);
+int64_t skv_fwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D);
 int launch_skv_bwd(const SkvAttnArgs &a, hipStream_t st);        // io_dtype QFA_F16, Nq <= 32: one fused pass
 int launch_skv_bwd_long(const SkvAttnArgs &a, hipStream_t st);   // io_dtype QFA_F16, any Nq: dQ kernel + dKV kernel
 

@@ -40,6 +40,9 @@ struct SkvArgs {
   float sm_scale_log2;
   int qblocks;   // query blocks per (batch, head)
   int BH;        // batch * heads
+  int splits;    // workgroups sharing the keys of one query block (1: the result goes straight to o / lse)
+  int tiles_per_split;
+  float *partial;   // splits > 1: [BH][qblocks][splits][16*D + 32] floats (O^T unnormalised, m in log2 units, l)
 };
 
 constexpr int SKV_NBUF = 3;
@@ -57,8 +60,10 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
 
   // block id -> (batch*head, query block): the query blocks of one (batch, head) get ids that differ
   // by 8, i.e. run on the same XCD close in time, and share its L2 copy of the codes
-  const int bh = (int)(blockIdx.x / (8 * a.qblocks)) * 8 + (int)(blockIdx.x % 8);
+  const int per_bh = a.qblocks * a.splits;
+  const int bh = (int)(blockIdx.x / (8 * per_bh)) * 8 + (int)(blockIdx.x % 8);
   const int qb = (int)(blockIdx.x / 8) % a.qblocks;
+  const int split = ((int)(blockIdx.x / 8) % per_bh) / a.qblocks;
   if (bh >= a.BH) return;
   const int64_t b = bh / a.H, h = bh % a.H;
   const int tid = threadIdx.x, lane = tid % 64, q16 = lane % 16, G = lane / 16;
@@ -67,13 +72,16 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
 
   const unsigned char *codes_bh = reinterpret_cast<const unsigned char *>(a.codes + b * a.scb + h * a.sch);
   const int64_t tk0 = (int64_t)bh * a.Nk, tq0 = (int64_t)bh * a.Nq;
-  const int ntiles = (a.Nk + SKV_TILE - 1) / SKV_TILE;
+  // this workgroup's tiles t0 .. t0 + ntiles - 1 (all of them unless the keys are split); wave w takes
+  // t0 + w, t0 + w + 4, ...
+  const int t0 = split * a.tiles_per_split;
+  const int ntiles = min(a.tiles_per_split, (a.Nk + SKV_TILE - 1) / SKV_TILE - t0);
   const int my_tiles = ntiles > wave ? (ntiles - wave + 3) / 4 : 0;
 
   Copy cp;
   cp.init((unsigned)a.scn, lane);
   auto issue = [&](int i, int slot_idx) {
-    const int t = wave + 4 * i;
+    const int t = t0 + wave + 4 * i;
     unsigned char *slot = smem + wave_off + slot_idx * SLOT;
     const int rows = min(SKV_TILE, a.Nk - t * SKV_TILE);
     const rsrc_t rs_k = make_rsrc(codes_bh + (int64_t)t * SKV_TILE * a.scn, (unsigned)((rows - 1) * (int)a.scn + D));
@@ -155,7 +163,7 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
     const unsigned char *slot = smem + slot_off;
     const unsigned *skp = reinterpret_cast<const unsigned *>(slot + K_BYTES);
     const unsigned *zpp = skp + SKV_TILE;
-    const int j0 = (wave + 4 * i) * SKV_TILE;
+    const int j0 = (t0 + wave + 4 * i) * SKV_TILE;
     u32x4 kw[2][(KS + 1) / 2];
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb)
@@ -244,7 +252,7 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
     } else {
       dma_wait();
     }
-    if ((wave + 4 * i + 1) * SKV_TILE > a.Nk) tile(i, cur, std::true_type{});
+    if ((t0 + wave + 4 * i + 1) * SKV_TILE > a.Nk) tile(i, cur, std::true_type{});
     else tile(i, cur, std::false_type{});
     cur = cur + 1 == SKV_NBUF ? 0 : cur + 1;
     nxt = nxt + 1 == SKV_NBUF ? 0 : nxt + 1;
@@ -270,7 +278,7 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
   }
   __syncthreads();
   if (wave == 0) {
-    float m_all = m_ref;   // finite: wave 0 always owns tile 0
+    float m_all = m_ref;   // finite: wave 0 always owns the first tile
 #pragma unroll
     for (int w = 0; w < 3; ++w) m_all = fmaxf(m_all, mg[w * MG + 16 * D + q16]);
     const float s0 = __builtin_amdgcn_exp2f(a_s * (m_ref - m_all));
@@ -280,6 +288,24 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
     for (int w = 0; w < 3; ++w) {
       sw[w] = __builtin_amdgcn_exp2f(a_s * (mg[w * MG + 16 * D + q16] - m_all));   // -inf for a wave without tiles
       l_all += mg[w * MG + 16 * D + 16 + q16] * sw[w];
+    }
+    if (a.splits > 1) {   // hand the unnormalised block result to the merge kernel
+      float *dst = a.partial + ((int64_t)(bh * a.qblocks + qb) * a.splits + split) * MG;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int d = 16 * db + 4 * G + v;
+          float acc = (oacc[db][v] - w_tot) * s0;
+#pragma unroll
+          for (int w = 0; w < 3; ++w) acc += mg[w * MG + d * 16 + q16] * sw[w];
+          dst[d * 16 + q16] = acc;
+        }
+      if (G == 0) {
+        dst[16 * D + q16] = a_s * m_all;
+        dst[16 * D + 16 + q16] = l_all;
+      }
+      return;
     }
     const float inv = 1.0f / l_all;
     if (qi < a.Nq) {
@@ -305,6 +331,52 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
   }
 }
 
+// Sum of the `splits` partial results of every query block: O = sum_s O_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).
+// One workgroup per (batch*head, query block); thread = (query tid%16, columns tid/16 + 16k).
+template <typename T, int D> __global__ __launch_bounds__(256) void skv_merge_kernel(SkvArgs a) {
+  constexpr int MG = 16 * D + 32;
+  const int bh = blockIdx.x / a.qblocks, qb = blockIdx.x % a.qblocks;
+  const int64_t b = bh / a.H, h = bh % a.H;
+  const int q16 = threadIdx.x % 16, dg = threadIdx.x / 16;
+  const int qi = 16 * qb + q16;
+  const float *src = a.partial + (int64_t)blockIdx.x * a.splits * MG;
+  float m = -INFINITY;
+  for (int s = 0; s < a.splits; ++s) m = fmaxf(m, src[s * MG + 16 * D + q16]);
+  float l = 0.f, acc[D / 16];
+#pragma unroll
+  for (int k = 0; k < D / 16; ++k) acc[k] = 0.f;
+  for (int s = 0; s < a.splits; ++s) {
+    const float w = __builtin_amdgcn_exp2f(src[s * MG + 16 * D + q16] - m);
+    l += src[s * MG + 16 * D + 16 + q16] * w;
+#pragma unroll
+    for (int k = 0; k < D / 16; ++k) acc[k] += src[s * MG + (dg + 16 * k) * 16 + q16] * w;
+  }
+  if (qi >= a.Nq) return;
+  const float inv = 1.0f / l;
+  T *orow = reinterpret_cast<T *>(a.o) + b * a.sob + h * a.soh + (int64_t)qi * a.son;
+#pragma unroll
+  for (int k = 0; k < D / 16; ++k) orow[dg + 16 * k] = (T)(acc[k] * inv);
+  if (dg == 0) a.lse[(int64_t)bh * a.Nq + qi] = (m + __log2f(l)) * kLn2;
+}
+
+// How the keys of one query block are split over workgroups: enough workgroups to fill the chip
+// (about four per CU), never fewer than 8 tiles per workgroup; 1 = no split.
+static void skv_split_plan(int64_t BH, int64_t Nq, int64_t Nk, int *splits, int *tiles_per_split) {
+  const int64_t ntiles = (Nk + SKV_TILE - 1) / SKV_TILE, wgs = BH * ((Nq + 15) / 16);
+  int64_t want = wgs >= 512 ? 1 : (1024 + wgs - 1) / wgs;
+  if (want > ntiles / 8) want = ntiles / 8;
+  if (want < 1) want = 1;
+  const int64_t tps = (ntiles + want - 1) / want;
+  *tiles_per_split = (int)tps;
+  *splits = (int)((ntiles + tps - 1) / tps);
+}
+
+int64_t skv_fwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D) {
+  int splits, tps;
+  skv_split_plan(B * H, Nq, Nk, &splits, &tps);
+  return splits > 1 ? B * H * ((Nq + 15) / 16) * splits * (int64_t)(16 * D + 32) * 4 : 0;
+}
+
 template <typename T, typename S, int D> static int launch_skv_fwd_tsd(const SkvAttnArgs &x, hipStream_t st) {
   SkvArgs a;
   a.q = x.q; a.codes = x.codes; a.scale = x.scale; a.zp = x.zp; a.o = x.o; a.lse = x.lse;
@@ -315,10 +387,22 @@ template <typename T, typename S, int D> static int launch_skv_fwd_tsd(const Skv
   if (x.B * x.H > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "attn_fwd_shared_kv: too many (batch, head) pairs");
   a.BH = (int)(x.B * x.H);
   a.qblocks = (int)((x.Nq + 15) / 16);
-  const int64_t total = (int64_t)a.qblocks * ((a.BH + 7) / 8) * 8;   // ids past batch*heads exit at once
+  a.splits = 1;
+  a.tiles_per_split = (int)((x.Nk + SKV_TILE - 1) / SKV_TILE);
+  a.partial = nullptr;
+  if (x.workspace) {   // validated: large enough for the plan below
+    skv_split_plan(x.B * x.H, x.Nq, x.Nk, &a.splits, &a.tiles_per_split);
+    a.partial = static_cast<float *>(x.workspace);
+  }
+  const int64_t total = (int64_t)a.qblocks * a.splits * ((a.BH + 7) / 8) * 8;   // ids past batch*heads exit at once
   if (total > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "attn_fwd_shared_kv: too many query blocks for one launch");
   skv_fwd_kernel<T, S, D><<<dim3((unsigned)total), dim3(256), 0, st>>>(a);
-  return check_launch("qfa_attn_fwd_shared_kv");
+  if (int e = check_launch("qfa_attn_fwd_shared_kv")) return e;
+  if (a.splits > 1) {
+    skv_merge_kernel<T, D><<<dim3((unsigned)(a.BH * a.qblocks)), dim3(256), 0, st>>>(a);
+    return check_launch("qfa_attn_fwd_shared_kv (merge)");
+  }
+  return 0;
 }
 
 template <typename T, int D> static int launch_skv_fwd_td(const SkvAttnArgs &x, hipStream_t st) {

@@ -148,12 +148,16 @@ def attn_fwd_shared_kv(q: torch.Tensor, codes: torch.Tensor, scale: torch.Tensor
     q, codes = _rows16(q), _rows16(codes)
     o = torch.empty((B, H, Nq, D), dtype=q.dtype, device=q.device)
     lse = torch.empty((B, H, Nq), dtype=torch.float32, device=q.device)
+    # scratch for the split over keys the library uses when B*H alone cannot fill the GPU (0: no split)
+    ws_bytes = _lib.lib().qfa_attn_fwd_shared_kv_workspace_bytes(B, H, Nq, Nk, D)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes > 0 else None
     with torch.cuda.device(q.device):
         code = _lib.lib().qfa_attn_fwd_shared_kv(
             q.data_ptr(), codes.data_ptr(), scale.data_ptr(), _lib.DTYPE_CODE[scale.dtype], zero_point.data_ptr(),
             o.data_ptr(), lse.data_ptr(), _lib.DTYPE_CODE[q.dtype], B, H, Nq, Nk, D,
             q.stride(0), q.stride(1), q.stride(2), codes.stride(0), codes.stride(1), codes.stride(2),
-            o.stride(0), o.stride(1), o.stride(2), float(sm_scale), _lib.stream_of(q))
+            o.stride(0), o.stride(1), o.stride(2), float(sm_scale),
+            workspace.data_ptr() if workspace is not None else None, ws_bytes, _lib.stream_of(q))
     _lib.check(code, "qfa_attn_fwd_shared_kv")
     return o, lse
 

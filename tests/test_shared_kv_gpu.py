@@ -130,6 +130,34 @@ def test_shared_kv_entry_point_long_query_block(qfa):
     assert_close("dKV", kvd.grad.cpu(), dkv_ref, scaled=True)
 
 
+@pytest.mark.parametrize("B,H,Nq,Nk,D", [(1, 2, 16, 4096, 128), (1, 1, 1, 20000, 64), (2, 3, 40, 3001, 128), (1, 8, 5, 1023, 64)])
+def test_shared_kv_forward_split_over_keys(qfa, B, H, Nq, Nk, D):
+    """Few (batch, head) pairs: the wrapper hands the library a workspace and the keys of a query block are
+    split over several workgroups, merged by a second kernel.  Same oracle, same bars; and the split result
+    agrees with the unsplit one (workspace = NULL) to a rounding of the output."""
+    from quant_flash_attn_amd import _lib
+    assert _lib.lib().qfa_attn_fwd_shared_kv_workspace_bytes(B, H, Nq, Nk, D) > 0
+    assert _lib.lib().qfa_attn_fwd_shared_kv_workspace_bytes(512, 16, 16, 3000, 128) == 0
+    q, kv = _inputs("normal", B, H, Nq, Nk, D, torch.float16, seed=Nk)
+    sm = 1.0 / math.sqrt(D)
+    codes, scale, zp = qfa.asymmetric_quant_per_token(kv.to(DEV))
+    qd = q.to(DEV)
+    o, lse = qfa.attn_fwd_shared_kv(qd, codes, scale, zp, sm)
+    o1 = torch.empty_like(o)
+    lse1 = torch.empty_like(lse)
+    s3 = lambda t: (t.stride(0), t.stride(1), t.stride(2))
+    rc = _lib.lib().qfa_attn_fwd_shared_kv(qd.data_ptr(), codes.data_ptr(), scale.data_ptr(), _lib.QFA_F16, zp.data_ptr(),
+                                           o1.data_ptr(), lse1.data_ptr(), _lib.QFA_F16, B, H, Nq, Nk, D, *s3(qd), *s3(codes),
+                                           *s3(o1), sm, None, 0, _lib.stream_of(qd))
+    assert rc == 0
+    torch.cuda.synchronize()
+    o_ref, lse_ref = oracle.legacy_fwd(q, codes.cpu(), scale.cpu(), zp.cpu(), sm)
+    assert_close("O", o.cpu(), o_ref, scaled=True)
+    assert max_abs(lse.cpu(), lse_ref) < LSE_TOL
+    assert max_abs(o.cpu(), o1.cpu()) <= 2.0 ** -9 * max(1.0, float(o_ref.abs().max()))
+    assert max_abs(lse.cpu(), lse1.cpu()) < 1e-4
+
+
 def test_shared_kv_offsets_cancel(qfa):
     """Every token with the same nonzero codes and extreme zero points: the 1152-offset terms the
     kernel adds to make the codes binary16 operands are orders of magnitude above the result and
