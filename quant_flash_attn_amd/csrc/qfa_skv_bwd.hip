@@ -68,8 +68,10 @@ template <int CPR> __device__ __forceinline__ int row_swizzle(int i) {
 
 template <int OFF> __device__ __forceinline__ u32x2 lds_tr16(unsigned addr) { return lds_read_tr16_async<OFF>(addr); }
 
-// S: element type of the scale vector (float or _Float16)
-template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_bwd_kernel(SkvBwdArgs a) {
+// S: element type of the scale vector (float or _Float16).  HALF: at most 16 queries -- rows 16..31 of the
+// query block are padding, so their share of steps 2 and 4 is skipped (P and dS are zero there).
+template <typename S, int D, bool HALF> __global__ __launch_bounds__(256, 2) void skv_bwd_kernel(SkvBwdArgs a) {
+  constexpr int QH = HALF ? 1 : 2;   // 16-query halves of the block that hold queries
   typedef SkvBwdSmem<D> SM;
   typedef Swz<D> KSW;
   typedef TileCopy<D, SKV_TILE, 64, KSW> Copy;
@@ -267,7 +269,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_bwd_k
     const float a_sk = key_ok ? a_s * sk : 0.f;
     const float sm_k = key_ok ? a.sm_scale : 0.f;   // a key past the end contributes nothing
 #pragma unroll
-    for (int aa = 0; aa < 4; ++aa) {
+    for (int aa = 0; aa < 2 * QH; ++aa) {
       const f32x4 l4 = *reinterpret_cast<const f32x4 *>(stat + 8 * aa + 4 * g);
       const f32x4 d4 = *reinterpret_cast<const f32x4 *>(stat + 32 + 8 * aa + 4 * g);
       float p[4], ds[4];
@@ -300,6 +302,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_bwd_k
       lds_wait_all();
       x0 = tie(x0);
       x1 = tie(x1);
+      if (HALF && G % 2 == 1) x0 = x1 = u32x2{0u, 0u};   // lanes of queries 16..31: nothing was written for them
       const u32x4 xb = {x0[0], x0[1], x1[0], x1[1]};
       const unsigned zc[4] = {magic_zp_pair(z0[0], z0[1]), magic_zp_pair(z0[2], z0[3]), magic_zp_pair(z1[0], z1[1]),
                               magic_zp_pair(z1[2], z1[3])};
@@ -327,7 +330,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_bwd_k
     for (int db = 0; db < DB; ++db) {
       u32x2 fr[2][2][2];   // [matrix: dO, Q][hh][r]
 #pragma unroll
-      for (int hh = 0; hh < 2; ++hh)
+      for (int hh = 0; hh < QH; ++hh)
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
           const unsigned ad = qt_off[hh][r] ^ ((4 * db) << 4);
@@ -339,7 +342,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_bwd_k
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 #pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
+      for (int hh = 0; hh < QH; ++hh) {
         const u32x2 d0 = tie(fr[0][hh][0]), d1 = tie(fr[0][hh][1]), q0 = tie(fr[1][hh][0]), q1 = tie(fr[1][hh][1]);
         acc = mfma_h(u32x4{d0[0], d0[1], d1[0], d1[1]}, pf[hh], acc);
         acc = mfma_h(u32x4{q0[0], q0[1], q1[0], q1[1]}, df[hh], acc);
@@ -422,7 +425,8 @@ template <typename S, int D> static int launch_skv_bwd_sd(const SkvAttnArgs &x, 
   a.sm_scale_log2 = x.sm_scale * kLog2e;
   const int64_t total = x.B * x.H;
   if (total > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "attn_bwd_shared_kv: too many (batch, head) pairs for one launch");
-  skv_bwd_kernel<S, D><<<dim3((unsigned)total), dim3(256), 0, st>>>(a);
+  if (x.Nq <= 16) skv_bwd_kernel<S, D, true><<<dim3((unsigned)total), dim3(256), 0, st>>>(a);
+  else skv_bwd_kernel<S, D, false><<<dim3((unsigned)total), dim3(256), 0, st>>>(a);
   return check_launch("qfa_attn_bwd_shared_kv");
 }
 
