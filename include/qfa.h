@@ -105,7 +105,7 @@ int qfa_attn_fwd(const int8_t *qc, const float *sq, const int8_t *zq, const int3
  *          to binary16), strides sq?, so?;  lse float [B*H*Nq]
  *   codes  int8 [B,H,Nk,D], strides sc?;  zp int8 [B*H*Nk]
  *   scale  [B*H*Nk] of scale_dtype: QFA_F32, or the same 16-bit type as io_dtype
- *   D in {64, 128}.  q, codes, o 16-byte aligned, strides multiples of 16 bytes, scn < 2^23.
+ *   D in {64, 128, 256}.  q, codes, o 16-byte aligned, strides multiples of 16 bytes, scn < 2^23.
  *   The sum of a query's D elements must stay inside binary16 range (|sum| < 65504).
  *   workspace  nullable.  With few (batch, head) pairs one workgroup per 16 queries leaves most of the
  *              chip idle (the reference launches one program per (batch, head)); given a caller-owned
@@ -132,7 +132,7 @@ int qfa_attn_fwd_shared_kv(const void *q, const int8_t *codes, const void *scale
  * writes each dKV row once); longer query blocks run a dQ kernel (one workgroup per 16 queries) and
  * a dKV kernel (one workgroup per 128 keys walking over the queries).
  *   q, o, dout, dq [B,H,Nq,D] and dkv [B,H,Nk,D] fp16 (io_dtype must be QFA_F16), strides as given;
- *   codes, scale, scale_dtype, zp, lse as in the forward.  D in {64, 128}.
+ *   codes, scale, scale_dtype, zp, lse as in the forward.  D in {64, 128, 256} (256: always the two kernels).
  *   The sums of a query's and of a dO row's D elements must stay inside binary16 range.
  */
 int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp,

@@ -1,12 +1,11 @@
 """Throughput report in the reference's own terms.
 
 Mirrors the two benchmark scripts of the reference on this build's entry points:
-  * compute_flops.py:89-168   Z=512, H=16, N_CTX_Q=16, N_CTX_KV=3000, HEAD_DIM in {64, 128}, fp16:
+  * compute_flops.py:89-168   Z=512, H=16, N_CTX_Q=16, N_CTX_KV=3000, HEAD_DIM in {64, 128, 256}, fp16:
                               forward and (fwd+bwd - fwd) backward time, TFLOP/s from
                               4*Z*H*Nq*Nkv*D (backward 2.5x, :103-104) and GB/s from the theoretical
                               traffic of calculate_theoretical_io (:39-83, 'quantized' provider);
   * test_speed.py:37-60       Z=256, H=16, N_CTX_Q=16, HEAD_DIM=128, N_CTX_KV in {512..4096}.
-HEAD_DIM=256 of the reference's sweep is left out (the attention kernels support 64 and 128).
 The comparison line is torch's scaled_dot_product_attention on the same fp16 tensors (the reference
 compares with the flash_attn package, which is not installed here).
 
@@ -62,6 +61,7 @@ def measure(Z, H, Nq, Nkv, D, provider, warmup=5, rep=20, dtype=torch.float16):
         fwd = lambda: quant_flash_attn(q, kv, kv_quant, sm)                                      # noqa: E731
     else:
         fwd = lambda: torch.nn.functional.scaled_dot_product_attention(q, kv, kv, scale=sm)    # noqa: E731
+    flops = 4.0 * Z * H * Nq * Nkv * D
     ms_fwd = _time(lambda: fwd(), warmup, rep)
     go = torch.randn((Z, H, Nq, D), dtype=dtype, device=dev)
 
@@ -71,7 +71,6 @@ def measure(Z, H, Nq, Nkv, D, provider, warmup=5, rep=20, dtype=torch.float16):
         fwd().backward(go)
 
     ms_bwd = max(_time(fwd_bwd, warmup, rep) - ms_fwd, 1e-6)
-    flops = 4.0 * Z * H * Nq * Nkv * D
     return {"Time Fwd (ms)": ms_fwd, "TFLOP/s Fwd": flops / (ms_fwd * 1e-3) / 1e12,
             "BW Fwd (GB/s)": theoretical_io(Z, H, Nq, Nkv, D, provider, "fwd") / (ms_fwd * 1e-3) / 1e9,
             "Time Bwd (ms)": ms_bwd, "TFLOP/s Bwd": 2.5 * flops / (ms_bwd * 1e-3) / 1e12,
@@ -98,7 +97,7 @@ def main(argv=None):
         sys.exit("compute_flops: needs a GPU")
     out = {}
     names = {"quantized": "this build (INT8 KV, libqfa)", "fp16": "torch SDPA (FP16)"}
-    for D in (64, 128):
+    for D in (64, 128, 256):
         Z, H, Nq, Nkv = (64 if args.small else 512), 16, 16, 3000
         rows = [(names[p], measure(Z, H, Nq, Nkv, D, p)) for p in ("quantized", "fp16")]
         _table(f"Z={Z} H={H} N_CTX_Q={Nq} N_CTX_KV={Nkv} HEAD_DIM={D} fp16", rows)

@@ -128,7 +128,8 @@ static int check_shared_kv(const char *who, const SkvAttnArgs &a) {
     return set_error(QFA_EINVAL, "%s: scale_dtype must be QFA_F32 or equal to io_dtype", who);
   if (a.B <= 0 || a.H <= 0 || a.Nq <= 0 || a.Nk <= 0) return set_error(QFA_EINVAL, "%s: B, H, Nq, Nk must be positive", who);
   if (a.Nq > 0x7fffff00LL || a.Nk > 0x7fffff00LL) return set_error(QFA_EUNSUPPORTED, "%s: sequence too long", who);
-  if (a.D != 64 && a.D != 128) return set_error(QFA_EUNSUPPORTED, "%s: head_dim %d not in {64, 128}", who, a.D);
+  if (a.D != 64 && a.D != 128 && a.D != 256)
+    return set_error(QFA_EUNSUPPORTED, "%s: head_dim %d not in {64, 128, 256}", who, a.D);
   if (!(a.sm_scale > 0.0f) || !(a.sm_scale < 3.0e38f))
     return set_error(QFA_EINVAL, "%s: sm_scale must be a positive finite number", who);
   if (!aligned16(a.q) || !aligned16(a.codes) || !aligned16(a.o))
@@ -141,7 +142,7 @@ static int check_shared_kv(const char *who, const SkvAttnArgs &a) {
 }
 
 int64_t qfa_attn_fwd_shared_kv_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D) {
-  if (B <= 0 || H <= 0 || Nq <= 0 || Nk <= 0 || (D != 64 && D != 128)) return 0;
+  if (B <= 0 || H <= 0 || Nq <= 0 || Nk <= 0 || (D != 64 && D != 128 && D != 256)) return 0;
   return skv_fwd_workspace_bytes(B, H, Nq, Nk, D);
 }
 
@@ -190,7 +191,8 @@ int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale
     return set_error(QFA_EINVAL, "%s: dout, dq, dkv must be 16-byte aligned", who);
   if (!strides_ok(sdob, sdoh, sdon, D, 2) || !strides_ok(sdqb, sdqh, sdqn, D, 2) || !strides_ok(sdkb, sdkh, sdkn, D, 2))
     return set_error(QFA_EINVAL, "%s: strides must be positive multiples of 16 bytes, token stride >= D", who);
-  return Nq <= 32 ? launch_skv_bwd(a, (hipStream_t)stream) : launch_skv_bwd_long(a, (hipStream_t)stream);
+  // one fused pass keeps a (batch, head)'s dQ in registers: at most 32 queries, head_dim up to 128
+  return Nq <= 32 && D <= 128 ? launch_skv_bwd(a, (hipStream_t)stream) : launch_skv_bwd_long(a, (hipStream_t)stream);
 }
 
 int qfa_bench_qk_stage(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,

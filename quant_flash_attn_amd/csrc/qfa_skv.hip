@@ -45,14 +45,15 @@ struct SkvArgs {
   float *partial;   // splits > 1: [BH][qblocks][splits][16*D + 32] floats (O^T unnormalised, m in log2 units, l)
 };
 
-constexpr int SKV_NBUF = 3;
+// ring depth per wave: three tiles, two at D = 256 (8 KB tiles)
+template <int D> constexpr int skv_nbuf() { return D == 256 ? 2 : 3; }
 
 template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) void skv_fwd_kernel(SkvArgs a) {
   typedef SwzSkv<D> KSW;
   typedef TileCopy<D, SKV_TILE, 64, KSW> Copy;
   constexpr int KS = D / 32;     // 32-wide k-steps of the score product
   constexpr int DB = D / 16;     // 16-row blocks of O^T
-  constexpr int OPS = Copy::N + 2;
+  constexpr int OPS = Copy::N + 2, SKV_NBUF = skv_nbuf<D>();
   constexpr int K_BYTES = SKV_TILE * D, SLOT = K_BYTES + 2 * SKV_TILE * 4, WAVE = SKV_NBUF * SLOT;
   constexpr int MG = 16 * D + 32;   // floats of one partial result: O^T [D][16], m[16], l[16]
   static_assert(3 * MG * 4 <= 4 * WAVE, "the merge area overlays the rings");
@@ -164,24 +165,28 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
     const unsigned *skp = reinterpret_cast<const unsigned *>(slot + K_BYTES);
     const unsigned *zpp = skp + SKV_TILE;
     const int j0 = (t0 + wave + 4 * i) * SKV_TILE;
-    u32x4 kw[2][(KS + 1) / 2];
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-      for (int mm = 0; mm < (KS + 1) / 2; ++mm)
-        kw[rb][mm] = *reinterpret_cast<const u32x4 *>(slot + (k_off[rb] ^ ((4 * mm) << 4)));
     const unsigned z_a[2] = {zpp[q16], zpp[16 + q16]};
-    u32x2 vr[DB];
+    // (the per-block read addresses are re-formed from these three every tile: one XOR each, instead of
+    // two dozen registers held across the loop)
+    int vt = vt_off, ko[2] = {k_off[0], k_off[1]};
+    asm volatile("" : "+v"(vt), "+v"(ko[0]), "+v"(ko[1]));
+    // transposed fragments for P.V in groups of 8 blocks (one group, two at D = 256), the first one now
+    constexpr int VG = DB < 8 ? DB : 8;
+    u32x2 vr[VG];
 #pragma unroll
-    for (int db = 0; db < DB; ++db) vr[db] = lds_read_tr8_async(lds0 + slot_off + (vt_off ^ (db << 4)));
+    for (int db = 0; db < VG; ++db) vr[db] = lds_read_tr8_async(lds0 + slot_off + (vt ^ (db << 4)));
     // ---- scores: two 16-key row blocks
     f32x4 f[2];
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) {
       f[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+      u32x4 kw[(KS + 1) / 2];
+#pragma unroll
+      for (int mm = 0; mm < (KS + 1) / 2; ++mm)
+        kw[mm] = *reinterpret_cast<const u32x4 *>(slot + (ko[rb] ^ ((4 * mm) << 4)));
 #pragma unroll
       for (int m = 0; m < KS; ++m)
-        f[rb] = mfma_h16(expand_codes(kw[rb][m / 2][2 * (m % 2)], kw[rb][m / 2][2 * (m % 2) + 1]), qf[m], f[rb]);
+        f[rb] = mfma_h16(expand_codes(kw[m / 2][2 * (m % 2)], kw[m / 2][2 * (m % 2) + 1]), qf[m], f[rb]);
       const unsigned cz = magic_zp_pair(z_a[rb], z_a[rb]);
       u32x4 corr_k = {0u, 0u, 0u, 0u};
       if (G == 0) {
@@ -236,11 +241,18 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
         w_run = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pp), __builtin_bit_cast(f16x2, cpair), w_run, false);
       }
     // ---- O^T += (1152 + codes)^T . P'^T, one k-step of 32 keys
-    lds_wait_all();
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const u32x2 w = tie(vr[db]);
-      oacc[db] = mfma_h16(expand_codes(w[0], w[1]), pf, oacc[db]);
+    for (int g0 = 0; g0 < DB; g0 += VG) {
+      lds_wait_all();
+      u32x2 cur[VG];
+#pragma unroll
+      for (int db = 0; db < VG; ++db) cur[db] = tie(vr[db]);
+      if (g0 + VG < DB) {
+#pragma unroll
+        for (int db = 0; db < VG; ++db) vr[db] = lds_read_tr8_async(lds0 + slot_off + (vt ^ ((g0 + VG + db) << 4)));
+      }
+#pragma unroll
+      for (int db = 0; db < VG; ++db) oacc[g0 + db] = mfma_h16(expand_codes(cur[db][0], cur[db][1]), pf, oacc[g0 + db]);
     }
   };
 
@@ -412,13 +424,15 @@ template <typename T, int D> static int launch_skv_fwd_td(const SkvAttnArgs &x, 
 
 int launch_skv_fwd(const SkvAttnArgs &x, hipStream_t st) {
   if (x.io_dtype == QFA_F16) {
+    if (x.D == 256) return launch_skv_fwd_td<_Float16, 256>(x, st);
     if (x.D == 128) return launch_skv_fwd_td<_Float16, 128>(x, st);
     if (x.D == 64) return launch_skv_fwd_td<_Float16, 64>(x, st);
   } else {
+    if (x.D == 256) return launch_skv_fwd_td<__bf16, 256>(x, st);
     if (x.D == 128) return launch_skv_fwd_td<__bf16, 128>(x, st);
     if (x.D == 64) return launch_skv_fwd_td<__bf16, 64>(x, st);
   }
-  return set_error(QFA_EUNSUPPORTED, "attn_fwd_shared_kv: head_dim must be 64 or 128");
+  return set_error(QFA_EUNSUPPORTED, "attn_fwd_shared_kv: head_dim must be 64, 128 or 256");
 }
 
 }  // namespace qfa

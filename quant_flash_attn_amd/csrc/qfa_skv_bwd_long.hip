@@ -13,6 +13,9 @@
 //                 registers) and the workgroup walks over the query blocks of 32, whose Q / dO / O rows
 //                 arrive in a double-buffered LDS area by direct global->LDS loads.  Every (tile, query
 //                 block) pair is visited once; each dKV row is written once, as whole 128-byte lines.
+//                 At D = 256 the accumulators of a tile do not fit one wave: two waves share a tile, each
+//                 keeping 128 of the 256 columns (both compute S and dP), a workgroup covers 64 keys and
+//                 the row area is single-buffered.
 // Both recompute delta from O and dO (no workspace), S and dP are computed in both kernels.
 #include <type_traits>
 
@@ -33,12 +36,12 @@ struct SkvBwdLongArgs {
 };
 
 // ------------------------------------------------------------------------------------------ dQ
-constexpr int SKVQ_NBUF = 3;
 
 template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dq_kernel(SkvBwdLongArgs a) {
   typedef SwzSkv<D> KSW;
   typedef TileCopy<D, SKV_TILE, 64, KSW> Copy;
   constexpr int KS = D / 32, DB = D / 16, OPS = Copy::N + 2;
+  constexpr int SKVQ_NBUF = D == 256 ? 2 : 3;   // ring depth per wave (8 KB tiles at D = 256)
   constexpr int K_BYTES = SKV_TILE * D, SLOT = K_BYTES + 2 * SKV_TILE * 4, WAVE = SKVQ_NBUF * SLOT;
   constexpr int MG = 16 * D;   // floats of one partial dQ^T [D][16]
   static_assert(3 * MG * 4 <= 4 * WAVE, "the merge area overlays the rings");
@@ -139,25 +142,28 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dq_ke
     const unsigned *skp = reinterpret_cast<const unsigned *>(slot + K_BYTES);
     const unsigned *zpp = skp + SKV_TILE;
     const int krem = a.Nk - (wave + 4 * i) * SKV_TILE;   // keys of this tile that exist (>= 32: all)
-    u32x4 kw[2][(KS + 1) / 2];
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-      for (int mm = 0; mm < (KS + 1) / 2; ++mm)
-        kw[rb][mm] = *reinterpret_cast<const u32x4 *>(slot + (k_off[rb] ^ ((4 * mm) << 4)));
     const unsigned z_a[2] = {zpp[q16], zpp[16 + q16]};
-    u32x2 vr[DB];
+    // (per-block read addresses are re-formed from these every tile: one XOR each instead of registers
+    // held across the loop)
+    int vt = vt_off, ko[2] = {k_off[0], k_off[1]};
+    asm volatile("" : "+v"(vt), "+v"(ko[0]), "+v"(ko[1]));
+    constexpr int VG = DB < 8 ? DB : 8;   // transposed fragments in groups of 8 blocks, the first one now
+    u32x2 vr[VG];
 #pragma unroll
-    for (int db = 0; db < DB; ++db) vr[db] = lds_read_tr8_async(lds0 + slot_off + (vt_off ^ (db << 4)));
+    for (int db = 0; db < VG; ++db) vr[db] = lds_read_tr8_async(lds0 + slot_off + (vt ^ (db << 4)));
     // ---- S^T and dP^T from the same expanded code operands
     f32x4 f[2], gq[2];
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) {
       f[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
       gq[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+      u32x4 kw[(KS + 1) / 2];
+#pragma unroll
+      for (int mm = 0; mm < (KS + 1) / 2; ++mm)
+        kw[mm] = *reinterpret_cast<const u32x4 *>(slot + (ko[rb] ^ ((4 * mm) << 4)));
 #pragma unroll
       for (int m = 0; m < KS; ++m) {
-        const u32x4 ca = expand_codes(kw[rb][m / 2][2 * (m % 2)], kw[rb][m / 2][2 * (m % 2) + 1]);
+        const u32x4 ca = expand_codes(kw[m / 2][2 * (m % 2)], kw[m / 2][2 * (m % 2) + 1]);
         f[rb] = mfma_h16(ca, qf[m], f[rb]);
         gq[rb] = mfma_h16(ca, dof[m], gq[rb]);
       }
@@ -193,11 +199,18 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dq_ke
       }
     }
     // ---- dQ^T += (1152 + codes)^T . x^T
-    lds_wait_all();
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const u32x2 w = tie(vr[db]);
-      acc[db] = mfma_h16(expand_codes(w[0], w[1]), xf, acc[db]);
+    for (int g0 = 0; g0 < DB; g0 += VG) {
+      lds_wait_all();
+      u32x2 now[VG];
+#pragma unroll
+      for (int db = 0; db < VG; ++db) now[db] = tie(vr[db]);
+      if (g0 + VG < DB) {
+#pragma unroll
+        for (int db = 0; db < VG; ++db) vr[db] = lds_read_tr8_async(lds0 + slot_off + (vt ^ ((g0 + VG + db) << 4)));
+      }
+#pragma unroll
+      for (int db = 0; db < VG; ++db) acc[g0 + db] = mfma_h16(expand_codes(now[db][0], now[db][1]), xf, acc[g0 + db]);
     }
   };
 
@@ -253,15 +266,17 @@ template <int D> struct RowSwz {
 };
 
 template <int D> struct SkvDkvSmem {
-  static constexpr int SLOT = SKV_TILE * D + 2 * SKV_TILE * 4;   // one tile per wave
+  static constexpr int DS = D == 256 ? 2 : 1;                    // waves sharing one tile (each keeps D / DS columns of dKV)
+  static constexpr int NRB = D == 256 ? 1 : 2;                   // row buffers
+  static constexpr int SLOT = SKV_TILE * D + 2 * SKV_TILE * 4;   // one tile copy per wave, used in the prologue only
   static constexpr int ROWS = 32 * D * 2;                        // one block of 32 binary16 rows
   static constexpr int BUF = 3 * ROWS;                           // Q, dO, O of one query block
-  static constexpr int OFF_BUF = 4 * SLOT;                       // two of them (double buffer)
-  static constexpr int OFF_STAT = OFF_BUF + 2 * BUF;             // per buffer: lse (log2), delta, rowsum(Q), rowsum(dO)
-  static constexpr int TOTAL = OFF_STAT + 2 * 4 * 32 * 4;
+  static constexpr int AREA = NRB * BUF > 4 * SLOT ? NRB * BUF : 4 * SLOT;   // rows overlay the tile copies
+  static constexpr int OFF_STAT = AREA;                          // per buffer: lse (log2), delta, rowsum(Q), rowsum(dO)
+  static constexpr int TOTAL = OFF_STAT + NRB * 4 * 32 * 4;
   static constexpr int STAGE = 32 * 128;                         // per wave, overlays the row buffers at the end
-  static_assert(4 * STAGE <= 2 * BUF, "the output stage overlays the row buffers");
-  static_assert(OFF_BUF % 256 == 0 && ROWS % 256 == 0, "row offsets are XOR-ed with block offsets");
+  static_assert(4 * STAGE <= AREA, "the output stage overlays the row buffers");
+  static_assert(ROWS % 256 == 0, "row offsets are XOR-ed with block offsets");
 };
 
 template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_kernel(SkvBwdLongArgs a) {
@@ -269,7 +284,8 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
   typedef Swz<D> KSW;
   typedef TileCopy<D, SKV_TILE, 64, KSW> Copy;
   typedef TileCopy<D * 2, 32, 256, RowSwz<D>> RowCopy;
-  constexpr int DB = D / 32, CPR = D / 8, KD = D / 16;
+  constexpr int DS = SM::DS, NRB = SM::NRB;
+  constexpr int DB = D / 32, DBW = DB / DS, CPR = D / 8, KD = D / 16;
   __shared__ __attribute__((aligned(256))) unsigned char smem[SM::TOTAL];
 
   const int bh = blockIdx.x / a.kchunks, chunk = blockIdx.x % a.kchunks;
@@ -277,7 +293,8 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
   const int tid = threadIdx.x, lane = tid % 64, lr = lane % 32, g = lane / 32;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int ntiles = (a.Nk + SKV_TILE - 1) / SKV_TILE;
-  const int t = 4 * chunk + wave;                 // this wave's tile
+  const int t = (4 / DS) * chunk + wave / DS;     // this wave's tile
+  const int db0 = (wave % DS) * DBW;              // first of its 32-column blocks of dKV
   const bool t_ok = t < ntiles;                   // (a wave without a tile still takes part in copies and barriers)
   const int j0 = t * SKV_TILE;
   const bool key_ok = j0 + lr < a.Nk;
@@ -292,7 +309,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
   co.init((unsigned)(a.son * 2), tid);
   const _Float16 *q_bh = a.q + b * a.sqb + h * a.sqh, *d_bh = a.dout + b * a.sdob + h * a.sdoh, *o_bh = a.o + b * a.sob + h * a.soh;
   auto issue_rows = [&](int qb) {
-    unsigned char *buf = smem + SM::OFF_BUF + (qb % 2) * SM::BUF;
+    unsigned char *buf = smem + (qb % NRB) * SM::BUF;
     const int rows = min(32, a.Nq - 32 * qb);
     // rows past Nq read as zeros (exact bounds)
     const rsrc_t rq = make_rsrc(q_bh + (int64_t)32 * qb * a.sqn, (unsigned)(((rows - 1) * (int)a.sqn + D) * 2));
@@ -313,7 +330,6 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
     skv_issue_tile<S, D>(cp, slot, reinterpret_cast<const unsigned char *>(a.codes + b * a.scb + h * a.sch), a.scale, a.zp,
                          tk0, t, a.Nk, a.scn, lane);
   }
-  issue_rows(0);
   dma_wait();
   u32x4 cb[KD];
   float sk = 0.f;
@@ -340,6 +356,8 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
   }
   const float a_sk = key_ok ? a.sm_scale_log2 * sk : 0.f;
   const float sm_k = key_ok ? a.sm_scale : 0.f;
+  __syncthreads();   // every wave has its operands in registers: the row buffers may overlay the tile copies
+  if (NRB == 2) issue_rows(0);
 
   // ---- per-lane LDS offsets inside a row block (as in the fused kernel)
   const unsigned lds0 = lds_addr(smem);
@@ -355,17 +373,21 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
       qt_off[hh][r] = i * (D * 2) + ((chk ^ RowSwz<D>::swz(i)) << 4) + 8 * (s16 % 2);
     }
 
-  f32x16 dkv[DB];
+  f32x16 dkv[DBW];
 #pragma unroll
-  for (int db = 0; db < DB; ++db)
+  for (int db = 0; db < DBW; ++db)
 #pragma unroll
     for (int v = 0; v < 16; ++v) dkv[db][v] = 0.f;
 
   for (int qb = 0; qb < nqb; ++qb) {
-    unsigned char *buf = smem + SM::OFF_BUF + (qb % 2) * SM::BUF;
-    float *stat = reinterpret_cast<float *>(smem + SM::OFF_STAT) + (qb % 2) * 128;
+    unsigned char *buf = smem + (qb % NRB) * SM::BUF;
+    float *stat = reinterpret_cast<float *>(smem + SM::OFF_STAT) + (qb % NRB) * 128;
+    if (NRB == 1) {
+      if (qb > 0) __syncthreads();   // everybody is done with block qb-1
+      issue_rows(qb);
+    }
     dma_wait();          // this thread's share of block qb has landed ...
-    __syncthreads();     // ... and everybody's; everybody is also done with block qb-1
+    __syncthreads();     // ... and everybody's; (two buffers:) everybody is also done with block qb-1
     // ---- delta, row sums, LSE of the block (thread = row tid/8, chunks tid%8 + {0, 8})
     {
       const int pi = tid / 8, part = tid % 8;
@@ -399,7 +421,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
         stat[96 + pi] = rd;
       }
     }
-    if (qb + 1 < nqb) issue_rows(qb + 1);   // the other buffer: nobody reads it any more
+    if (NRB == 2 && qb + 1 < nqb) issue_rows(qb + 1);   // the other buffer: nobody reads it any more
     __syncthreads();
     if (!t_ok) continue;
 
@@ -449,15 +471,15 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
       }
     }
     // ---- dKV^T += dO^T P + Q^T dS
-    const unsigned bufa = lds0 + SM::OFF_BUF + (qb % 2) * SM::BUF;
+    const unsigned bufa = lds0 + (qb % NRB) * SM::BUF;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
+    for (int db = 0; db < DBW; ++db) {
       u32x2 fr[2][2][2];   // [matrix: dO, Q][hh][r]
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
-          const unsigned ad = bufa + (qt_off[hh][r] ^ ((4 * db) << 4));
+          const unsigned ad = bufa + (qt_off[hh][r] ^ ((4 * (db0 + db)) << 4));
           fr[0][hh][r] = lds_read_tr16_async<SM::ROWS>(ad);
           fr[1][hh][r] = lds_read_tr16_async<0>(ad);
         }
@@ -474,12 +496,12 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
   // ---- the tile's dKV rows leave through an LDS stage as whole 128-byte lines (two 32-column blocks a time)
   __syncthreads();   // the row buffers are done with: the stages overlay them
   if (t_ok) {
-    unsigned char *stage = smem + SM::OFF_BUF + wave * SM::STAGE;
+    unsigned char *stage = smem + wave * SM::STAGE;
     _Float16 *dkv_bh = a.dkv + b * a.sdkb + h * a.sdkh;
     const int st_w = lr * 128 + 8 * g, st_wswz = lr % 8;
     const int st_r = (lane / 8) * 128 + (((lane % 8) ^ (lane / 8)) << 4);
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
+    for (int db = 0; db < DBW; ++db) {
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa) {
         u32x2 o2;
@@ -492,7 +514,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
         for (int it = 0; it < 4; ++it) {
           const u32x4 row16 = *reinterpret_cast<const u32x4 *>(stage + st_r + it * 1024);
           const int j = j0 + 8 * it + lane / 8;
-          if (j < a.Nk) *reinterpret_cast<u32x4 *>(dkv_bh + (int64_t)j * a.sdkn + 32 * (db - 1) + 8 * (lane % 8)) = row16;
+          if (j < a.Nk) *reinterpret_cast<u32x4 *>(dkv_bh + (int64_t)j * a.sdkn + 32 * (db0 + db - 1) + 8 * (lane % 8)) = row16;
         }
       }
     }
@@ -514,7 +536,8 @@ template <typename S, int D> static int launch_skv_bwd_long_sd(const SkvAttnArgs
   if (x.B * x.H > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "attn_bwd_shared_kv: too many (batch, head) pairs");
   a.BH = (int)(x.B * x.H);
   a.qblocks = (int)((x.Nq + 15) / 16);
-  a.kchunks = (int)((x.Nk + 4 * SKV_TILE - 1) / (4 * SKV_TILE));
+  const int keys_per_wg = 4 * SKV_TILE / SkvDkvSmem<D>::DS;
+  a.kchunks = (int)((x.Nk + keys_per_wg - 1) / keys_per_wg);
   const int64_t total_q = (int64_t)a.qblocks * ((a.BH + 7) / 8) * 8, total_k = (int64_t)a.kchunks * a.BH;
   if (total_q > 0x7fffffffLL || total_k > 0x7fffffffLL)
     return set_error(QFA_EUNSUPPORTED, "attn_bwd_shared_kv: too many blocks for one launch");
@@ -526,9 +549,10 @@ template <typename S, int D> static int launch_skv_bwd_long_sd(const SkvAttnArgs
 
 int launch_skv_bwd_long(const SkvAttnArgs &x, hipStream_t st) {
   const bool s32 = x.scale_dtype == QFA_F32;
+  if (x.D == 256) return s32 ? launch_skv_bwd_long_sd<float, 256>(x, st) : launch_skv_bwd_long_sd<_Float16, 256>(x, st);
   if (x.D == 128) return s32 ? launch_skv_bwd_long_sd<float, 128>(x, st) : launch_skv_bwd_long_sd<_Float16, 128>(x, st);
   if (x.D == 64) return s32 ? launch_skv_bwd_long_sd<float, 64>(x, st) : launch_skv_bwd_long_sd<_Float16, 64>(x, st);
-  return set_error(QFA_EUNSUPPORTED, "attn_bwd_shared_kv: head_dim must be 64 or 128");
+  return set_error(QFA_EUNSUPPORTED, "attn_bwd_shared_kv: head_dim must be 64, 128 or 256");
 }
 
 }  // namespace qfa

@@ -51,7 +51,8 @@ __device__ __forceinline__ f32x4 mfma_h16(u32x4 a, u32x4 b, f32x4 c) {
 template <int D> struct SwzSkv {
   static constexpr int CPR = D / 16;
   static __device__ __forceinline__ int swz(int row) {
-    return D == 128 ? ((row / 2) ^ ((row / 16) * 4)) % 8 : ((row / 4) ^ ((row / 16) * 2)) % 4;
+    return D == 256 ? (row ^ ((row / 16) * 4)) % 16
+           : D == 128 ? ((row / 2) ^ ((row / 16) * 4)) % 8 : ((row / 4) ^ ((row / 16) * 2)) % 4;
   }
 };
 

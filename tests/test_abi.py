@@ -66,7 +66,7 @@ def test_argument_errors_need_no_gpu(qfa):
         return L.qfa_attn_fwd_shared_kv(q, ok_ptr, ok_ptr, sdt, ok_ptr, ok_ptr, ok_ptr, io, 1, 1, Nq, Nk, D,
                                         *sq, *sc, *sq, sm, None, 0, None)
     assert skv_fwd(q=None) == -1 and b"null" in L.qfa_last_error()
-    assert skv_fwd(D=256) == -2 and b"head_dim" in L.qfa_last_error()
+    assert skv_fwd(D=96) == -2 and b"head_dim" in L.qfa_last_error()
     assert skv_fwd(io=0) == -1 and b"io_dtype" in L.qfa_last_error()
     assert skv_fwd(io=1, sdt=2) == -1 and b"scale_dtype" in L.qfa_last_error()
     assert skv_fwd(sm=float("nan")) == -1 and b"sm_scale" in L.qfa_last_error()

@@ -35,6 +35,9 @@ CASES = [
     (1, 2, 17, 1023, 128, "outlier", torch.float16, torch.float16),
     (1, 4, 32, 512, 64, "normal", torch.bfloat16, torch.bfloat16),
     (1, 2, 128, 4096, 128, "normal", torch.bfloat16, torch.float16),  # scale converted by the wrapper
+    (2, 2, 16, 3000, 256, "normal", torch.float16, torch.float16),    # head_dim 256 (compute_flops.py:94)
+    (1, 2, 37, 333, 256, "offset", torch.bfloat16, torch.float32),
+    (1, 1, 3, 9000, 256, "uniform", torch.float16, torch.float16),    # split over keys
 ]
 
 
@@ -67,6 +70,10 @@ BWD_CASES = [
     (1, 3, 33, 100, 64, "offset", torch.float32),        # one query past a block, one key chunk
     (1, 2, 128, 1000, 128, "uniform", torch.float16),
     (2, 2, 64, 129, 64, "outlier", torch.float32),       # second key chunk holds a single key
+    # head_dim 256 (compute_flops.py:94): always the two kernels, two waves share a tile in the dKV kernel
+    (2, 2, 16, 3000, 256, "normal", torch.float16),
+    (1, 2, 70, 161, 256, "offset", torch.float32),
+    (1, 1, 1, 1, 256, "normal", torch.float16),
 ]
 
 
