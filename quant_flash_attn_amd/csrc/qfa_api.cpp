@@ -191,6 +191,9 @@ int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale
     return set_error(QFA_EINVAL, "%s: dout, dq, dkv must be 16-byte aligned", who);
   if (!strides_ok(sdob, sdoh, sdon, D, 2) || !strides_ok(sdqb, sdqh, sdqn, D, 2) || !strides_ok(sdkb, sdkh, sdkn, D, 2))
     return set_error(QFA_EINVAL, "%s: strides must be positive multiples of 16 bytes, token stride >= D", who);
+  // the row copies of the two-kernel path form offsets inside a 32-row block in 31 bits
+  if (sqn >= (1 << 23) || son >= (1 << 23) || sdon >= (1 << 23))
+    return set_error(QFA_EUNSUPPORTED, "%s: token strides of 2^23 elements or more are not supported", who);
   // one fused pass keeps a (batch, head)'s dQ in registers: at most 32 queries, head_dim up to 128
   return Nq <= 32 && D <= 128 ? launch_skv_bwd(a, (hipStream_t)stream) : launch_skv_bwd_long(a, (hipStream_t)stream);
 }
