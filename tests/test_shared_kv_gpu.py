@@ -253,3 +253,39 @@ def test_shared_kv_graph_capture_and_replay(qfa, B, H, Nq, Nk):
             torch.cuda.synchronize()
             for name, a_, b_ in zip(("O", "LSE", "dQ", "dKV"), outs, eager):
                 assert torch.equal(a_, b_), f"graph replay differs from eager: {name} (round {rep})"
+
+
+@pytest.mark.parametrize("D", [128, 64])
+def test_shared_kv_full_benchmark_size(qfa, D):
+    """The reference's benchmark shape at full size (compute_flops.py:96: Z=512, H=16, 16 queries, 3000 keys):
+    sampled (batch, head) slices against the dense fp64 oracle, plus size-independent properties --
+    determinism (two runs bit-identical), softmax weights summing to one (a constant channel of kv comes out
+    of O as that constant), and a zero dO giving exactly zero gradients."""
+    Z, H, Nq, Nk = 512, 16, 16, 3000
+    g = torch.Generator(device=DEV).manual_seed(7)
+    q = torch.randn((Z, H, Nq, D), generator=g, device=DEV, dtype=torch.float16)
+    kv = torch.randn((Z, H, Nk, D), generator=g, device=DEV, dtype=torch.float16)
+    kv[..., 0] = 1.0                                   # a constant channel: O[..., 0] must be 1
+    do = torch.randn((Z, H, Nq, D), generator=g, device=DEV, dtype=torch.float16)
+    sm = 1.0 / math.sqrt(D)
+    codes, scale, zp = qfa.asymmetric_quant_per_token(kv)
+    del kv
+    o, lse = qfa.attn_fwd_shared_kv(q, codes, scale, zp, sm)
+    dq, dkv = qfa.attn_bwd_shared_kv(q, codes, scale, zp, o, do, lse, sm)
+    o2, lse2 = qfa.attn_fwd_shared_kv(q, codes, scale, zp, sm)
+    dq2, dkv2 = qfa.attn_bwd_shared_kv(q, codes, scale, zp, o, do, lse, sm)
+    torch.cuda.synchronize()
+    assert torch.equal(o, o2) and torch.equal(lse, lse2) and torch.equal(dq, dq2) and torch.equal(dkv, dkv2)
+    # the constant channel dequantizes to 1 up to one quantization step; softmax weights sum to one
+    kv0 = (codes[..., 0].float() - zp[..., 0].float()) * scale[..., 0].float()
+    assert float((o[..., 0].float() - 1.0).abs().max()) <= float((kv0 - 1.0).abs().max()) + 2.0 ** -9
+    dq0, dkv0 = qfa.attn_bwd_shared_kv(q, codes, scale, zp, o, torch.zeros_like(do), lse, sm)
+    assert float(dq0.abs().max()) == 0.0 and float(dkv0.abs().max()) == 0.0
+    for b, h in ((0, 0), (137, 5), (511, 15)):
+        sl = lambda t: t[b:b + 1, h:h + 1].cpu()
+        o_ref, lse_ref = oracle.legacy_fwd(sl(q), sl(codes), sl(scale), sl(zp), sm)
+        dq_ref, dkv_ref = oracle.legacy_bwd(sl(q), sl(codes), sl(scale), sl(zp), sl(do), sm)
+        assert_close(f"O[{b},{h}]", sl(o), o_ref, scaled=True)
+        assert max_abs(sl(lse), lse_ref) < LSE_TOL
+        assert_close(f"dQ[{b},{h}]", sl(dq), dq_ref, scaled=True)
+        assert_close(f"dKV[{b},{h}]", sl(dkv), dkv_ref, scaled=True)
