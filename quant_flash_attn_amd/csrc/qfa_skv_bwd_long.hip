@@ -268,15 +268,17 @@ template <int D> struct RowSwz {
 template <int D> struct SkvDkvSmem {
   static constexpr int DS = D == 256 ? 2 : 1;                    // waves sharing one tile (each keeps D / DS columns of dKV)
   static constexpr int NRB = D == 256 ? 1 : 2;                   // row buffers
+  static constexpr bool O_IN_LDS = NRB == 2;                     // one buffer: O (needed for delta only) is read from memory
   static constexpr int SLOT = SKV_TILE * D + 2 * SKV_TILE * 4;   // one tile copy per wave, used in the prologue only
   static constexpr int ROWS = 32 * D * 2;                        // one block of 32 binary16 rows
-  static constexpr int BUF = 3 * ROWS;                           // Q, dO, O of one query block
-  static constexpr int AREA = NRB * BUF > 4 * SLOT ? NRB * BUF : 4 * SLOT;   // rows overlay the tile copies
-  static constexpr int OFF_STAT = AREA;                          // per buffer: lse (log2), delta, rowsum(Q), rowsum(dO)
-  static constexpr int TOTAL = OFF_STAT + NRB * 4 * 32 * 4;
+  static constexpr int BUF = (O_IN_LDS ? 3 : 2) * ROWS;          // Q, dO (, O) of one query block
+  static constexpr int OFF_SLOT = NRB * BUF;                     // tile copies behind the row buffers: both are
+  static constexpr int OFF_STAT = OFF_SLOT + 4 * SLOT;           //   copied at once in the prologue
+  static constexpr int TOTAL = OFF_STAT + NRB * 4 * 32 * 4;      // per buffer: lse (log2), delta, rowsum(Q), rowsum(dO)
   static constexpr int STAGE = 32 * 128;                         // per wave, overlays the row buffers at the end
-  static_assert(4 * STAGE <= AREA, "the output stage overlays the row buffers");
+  static_assert(4 * STAGE <= NRB * BUF, "the output stage overlays the row buffers");
   static_assert(ROWS % 256 == 0, "row offsets are XOR-ed with block offsets");
+  static_assert(2 * TOTAL <= 160 * 1024, "two workgroups per CU");
 };
 
 template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_kernel(SkvBwdLongArgs a) {
@@ -298,7 +300,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
   const bool t_ok = t < ntiles;                   // (a wave without a tile still takes part in copies and barriers)
   const int j0 = t * SKV_TILE;
   const bool key_ok = j0 + lr < a.Nk;
-  unsigned char *slot = smem + wave * SM::SLOT;
+  unsigned char *slot = smem + SM::OFF_SLOT + wave * SM::SLOT;
   const int64_t tk0 = (int64_t)bh * a.Nk, tq0 = (int64_t)bh * a.Nq;
   const int nqb = (a.Nq + 31) / 32;
 
@@ -319,7 +321,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
     for (int c = 0; c < RowCopy::N; ++c) {
       cq.issue_one(rq, buf, wave, tid, c);
       cd.issue_one(rd, buf + SM::ROWS, wave, tid, c);
-      co.issue_one(ro, buf + 2 * SM::ROWS, wave, tid, c);
+      if (SM::O_IN_LDS) co.issue_one(ro, buf + 2 * SM::ROWS, wave, tid, c);
     }
   };
 
@@ -330,6 +332,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
     skv_issue_tile<S, D>(cp, slot, reinterpret_cast<const unsigned char *>(a.codes + b * a.scb + h * a.sch), a.scale, a.zp,
                          tk0, t, a.Nk, a.scn, lane);
   }
+  issue_rows(0);   // together with the tile: one memory latency for both
   dma_wait();
   u32x4 cb[KD];
   float sk = 0.f;
@@ -356,8 +359,6 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
   }
   const float a_sk = key_ok ? a.sm_scale_log2 * sk : 0.f;
   const float sm_k = key_ok ? a.sm_scale : 0.f;
-  __syncthreads();   // every wave has its operands in registers: the row buffers may overlay the tile copies
-  if (NRB == 2) issue_rows(0);
 
   // ---- per-lane LDS offsets inside a row block (as in the fused kernel)
   const unsigned lds0 = lds_addr(smem);
@@ -382,9 +383,19 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
   for (int qb = 0; qb < nqb; ++qb) {
     unsigned char *buf = smem + (qb % NRB) * SM::BUF;
     float *stat = reinterpret_cast<float *>(smem + SM::OFF_STAT) + (qb % NRB) * 128;
-    if (NRB == 1) {
-      if (qb > 0) __syncthreads();   // everybody is done with block qb-1
+    if (NRB == 1 && qb > 0) {
+      __syncthreads();   // everybody is done with block qb-1
       issue_rows(qb);
+    }
+    // (one buffer: O does not pass through LDS; this thread's chunks of it are fetched while the copy lands)
+    u32x4 og[SM::O_IN_LDS ? 1 : (CPR + 7) / 8];
+    if (!SM::O_IN_LDS) {
+      const int pi = tid / 8, part = tid % 8;
+      const bool live = 32 * qb + pi < a.Nq;
+#pragma unroll
+      for (int k = 0; k < (CPR + 7) / 8; ++k)
+        og[k] = live ? *reinterpret_cast<const u32x4 *>(o_bh + (int64_t)(32 * qb + pi) * a.son + (part + 8 * k) * 8)
+                     : u32x4{0u, 0u, 0u, 0u};
     }
     dma_wait();          // this thread's share of block qb has landed ...
     __syncthreads();     // ... and everybody's; (two buffers:) everybody is also done with block qb-1
@@ -397,7 +408,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
         const int off = pi * (D * 2) + ((c ^ RowSwz<D>::swz(pi)) << 4);
         const u32x4 qv = *reinterpret_cast<const u32x4 *>(buf + off);
         const u32x4 dv = *reinterpret_cast<const u32x4 *>(buf + SM::ROWS + off);
-        const u32x4 ov = *reinterpret_cast<const u32x4 *>(buf + 2 * SM::ROWS + off);
+        const u32x4 ov = SM::O_IN_LDS ? *reinterpret_cast<const u32x4 *>(buf + 2 * SM::ROWS + off) : og[c / 8];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const unsigned qw = qv[e], dw = dv[e], ow = ov[e];
@@ -496,7 +507,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
   // ---- the tile's dKV rows leave through an LDS stage as whole 128-byte lines (two 32-column blocks a time)
   __syncthreads();   // the row buffers are done with: the stages overlay them
   if (t_ok) {
-    unsigned char *stage = smem + wave * SM::STAGE;
+    unsigned char *stage = smem + wave * SM::STAGE;   // (row buffers)
     _Float16 *dkv_bh = a.dkv + b * a.sdkb + h * a.sdkh;
     const int st_w = lr * 128 + 8 * g, st_wswz = lr % 8;
     const int st_r = (lane / 8) * 128 + (((lane % 8) ^ (lane / 8)) << 4);
