@@ -289,3 +289,34 @@ def test_shared_kv_full_benchmark_size(qfa, D):
         assert max_abs(sl(lse), lse_ref) < LSE_TOL
         assert_close(f"dQ[{b},{h}]", sl(dq), dq_ref, scaled=True)
         assert_close(f"dKV[{b},{h}]", sl(dkv), dkv_ref, scaled=True)
+
+
+@pytest.mark.parametrize("Nq", [16, 48])
+def test_shared_kv_backward_strided_views(qfa, Nq):
+    """q, o, dO, the codes and the gradient buffers handed over as views of larger buffers (token stride
+    > D, [B,N,H,D] storage): same bits as with dense tensors, through the C entry point directly."""
+    from quant_flash_attn_amd import _lib
+    B, H, Nk, D = 2, 3, 300, 64
+    q, kv = _inputs("normal", B, H, Nq, Nk, D, torch.float16, seed=21)
+    do = torch.randn(q.shape, generator=torch.Generator().manual_seed(5)).to(torch.float16)
+    sm = 0.125
+    codes, scale, zp = qfa.asymmetric_quant_per_token(kv.to(DEV))
+    qd, dod = q.to(DEV), do.to(DEV)
+    o, lse = qfa.attn_fwd_shared_kv(qd, codes, scale, zp, sm)
+    dq, dkv = qfa.attn_bwd_shared_kv(qd, codes, scale, zp, o, dod, lse, sm)
+
+    def bnhd(t, pad):   # [B,N,H,D+pad] storage viewed as [B,H,N,D]
+        buf = torch.zeros((t.shape[0], t.shape[2], t.shape[1], t.shape[3] + pad), dtype=t.dtype, device=DEV)
+        view = buf.permute(0, 2, 1, 3)[..., :t.shape[3]]
+        view.copy_(t)
+        return view
+    q_v, o_v, do_v, c_v = bnhd(qd, 8), bnhd(o, 16), bnhd(dod, 0), bnhd(codes, 64)
+    dq_v, dkv_v = bnhd(torch.zeros_like(dq), 24), bnhd(torch.zeros_like(dkv), 8)
+    s3 = lambda t: (t.stride(0), t.stride(1), t.stride(2))
+    rc = _lib.lib().qfa_attn_bwd_shared_kv(
+        q_v.data_ptr(), c_v.data_ptr(), scale.data_ptr(), _lib.QFA_F16, zp.data_ptr(), o_v.data_ptr(), do_v.data_ptr(),
+        lse.data_ptr(), dq_v.data_ptr(), dkv_v.data_ptr(), _lib.QFA_F16, B, H, Nq, Nk, D,
+        *s3(q_v), *s3(c_v), *s3(o_v), *s3(do_v), *s3(dq_v), *s3(dkv_v), sm, _lib.stream_of(qd))
+    assert rc == 0, _lib.lib().qfa_last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(dq_v, dq) and torch.equal(dkv_v, dkv)
