@@ -30,7 +30,7 @@ struct SkvBwdLongArgs {
   const float *lse;
   _Float16 *dq, *dkv;
   int64_t H;
-  int Nq, Nk, BH, qblocks, kchunks;
+  int Nq, Nk, BH, qblocks, kchunks, cpw;   // cpw: key chunks per workgroup of the dKV kernel
   int64_t sqb, sqh, sqn, scb, sch, scn, sob, soh, son, sdob, sdoh, sdon, sdqb, sdqh, sdqn, sdkb, sdkh, sdkn;
   float sm_scale, sm_scale_log2;
 };
@@ -274,14 +274,23 @@ template <int D> struct SkvDkvSmem {
   static constexpr int BUF = (O_IN_LDS ? 3 : 2) * ROWS;          // Q, dO (, O) of one query block
   static constexpr int OFF_SLOT = NRB * BUF;                     // tile copies behind the row buffers: both are
   static constexpr int OFF_STAT = OFF_SLOT + 4 * SLOT;           //   copied at once in the prologue
-  static constexpr int TOTAL = OFF_STAT + NRB * 4 * 32 * 4;      // per buffer: lse (log2), delta, rowsum(Q), rowsum(dO)
-  static constexpr int STAGE = 32 * 128;                         // per wave, overlays the row buffers at the end
+  static constexpr int STAGE = 32 * 128;                         // per wave: 64 columns of its tile's dKV rows on their way out
+  // where the stages live while the rows stay resident: in the O rows (not needed after the statistics) when
+  // two stages fit one block of them, else in the tile slot when a stage fits it, else in an area of their own
+  static constexpr int STAGE_MODE = O_IN_LDS && 2 * STAGE <= ROWS ? 0 : (!O_IN_LDS && STAGE <= SLOT ? 2 : 1);
+  static constexpr int OFF_STAGE = OFF_STAT + NRB * 4 * 32 * 4;  // per buffer: lse (log2), delta, rowsum(Q), rowsum(dO)
+  static constexpr int TOTAL = OFF_STAGE + (STAGE_MODE == 1 ? 4 * STAGE : 0);
   static_assert(4 * STAGE <= NRB * BUF, "the output stage overlays the row buffers");
   static_assert(ROWS % 256 == 0, "row offsets are XOR-ed with block offsets");
   static_assert(2 * TOTAL <= 160 * 1024, "two workgroups per CU");
 };
 
-template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_kernel(SkvBwdLongArgs a) {
+// KEEP: all query blocks fit the row buffers (Nq <= 32 * NRB).  They are copied once, their statistics are
+// computed once, and the workgroup then walks over `cpw` consecutive 128-key chunks of its (batch, head)
+// with no barrier at all: each wave waits for its own tile copy, expands it into registers, puts the copy
+// of its next tile into the same slot, and computes.  Otherwise (longer query blocks) one workgroup per
+// chunk, the row blocks cycling through the buffers with two barriers a block.
+template <typename S, int D, bool KEEP> __global__ __launch_bounds__(256, 2) void skv_dkv_kernel(SkvBwdLongArgs a) {
   typedef SkvDkvSmem<D> SM;
   typedef Swz<D> KSW;
   typedef TileCopy<D, SKV_TILE, 64, KSW> Copy;
@@ -290,21 +299,21 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
   constexpr int DB = D / 32, DBW = DB / DS, CPR = D / 8, KD = D / 16;
   __shared__ __attribute__((aligned(256))) unsigned char smem[SM::TOTAL];
 
-  const int bh = blockIdx.x / a.kchunks, chunk = blockIdx.x % a.kchunks;
+  const int wgs_per_bh = (a.kchunks + a.cpw - 1) / a.cpw;
+  const int bh = blockIdx.x / wgs_per_bh;
+  const int c_begin = (blockIdx.x % wgs_per_bh) * a.cpw, c_end = min(a.kchunks, c_begin + a.cpw);
   const int64_t b = bh / a.H, h = bh % a.H;
   const int tid = threadIdx.x, lane = tid % 64, lr = lane % 32, g = lane / 32;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int ntiles = (a.Nk + SKV_TILE - 1) / SKV_TILE;
-  const int t = (4 / DS) * chunk + wave / DS;     // this wave's tile
-  const int db0 = (wave % DS) * DBW;              // first of its 32-column blocks of dKV
-  const bool t_ok = t < ntiles;                   // (a wave without a tile still takes part in copies and barriers)
-  const int j0 = t * SKV_TILE;
-  const bool key_ok = j0 + lr < a.Nk;
+  const int db0 = (wave % DS) * DBW;              // first of this wave's 32-column blocks of dKV
   unsigned char *slot = smem + SM::OFF_SLOT + wave * SM::SLOT;
+  const unsigned char *codes_bh = reinterpret_cast<const unsigned char *>(a.codes + b * a.scb + h * a.sch);
   const int64_t tk0 = (int64_t)bh * a.Nk, tq0 = (int64_t)bh * a.Nq;
   const int nqb = (a.Nq + 31) / 32;
+  auto tile_of = [&](int chunk) { return (4 / DS) * chunk + wave / DS; };   // this wave's tile in a chunk
 
-  // ---- row copies of a query block: Q, dO, O -> buffer (direct loads, 2 chunks per thread and matrix)
+  // ---- row copies of a query block: Q, dO (, O) -> buffer (direct loads)
   RowCopy cq, cd, co;
   cq.init((unsigned)(a.sqn * 2), tid);
   cd.init((unsigned)(a.sdon * 2), tid);
@@ -324,41 +333,56 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
       if (SM::O_IN_LDS) co.issue_one(ro, buf + 2 * SM::ROWS, wave, tid, c);
     }
   };
+  // delta, row sums, LSE of block qb from its buffer (thread = row tid/8, chunks tid%8 + 8k).  One buffer:
+  // O does not pass through LDS, `og` holds this thread's chunks of it.
+  auto block_stats = [&](int qb, const u32x4 *og) {
+    const unsigned char *buf = smem + (qb % NRB) * SM::BUF;
+    float *stat = reinterpret_cast<float *>(smem + SM::OFF_STAT) + (qb % NRB) * 128;
+    const int pi = tid / 8, part = tid % 8;
+    float dsum = 0.f, rq = 0.f, rd = 0.f;
+#pragma unroll
+    for (int c = part; c < CPR; c += 8) {
+      const int off = pi * (D * 2) + ((c ^ RowSwz<D>::swz(pi)) << 4);
+      const u32x4 qv = *reinterpret_cast<const u32x4 *>(buf + off);
+      const u32x4 dv = *reinterpret_cast<const u32x4 *>(buf + SM::ROWS + off);
+      const u32x4 ov = SM::O_IN_LDS ? *reinterpret_cast<const u32x4 *>(buf + 2 * SM::ROWS + off) : og[c / 8];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const unsigned qw = qv[e], dw = dv[e], ow = ov[e];
+        const float d0 = lo_to_f32<_Float16>(dw), d1 = hi_to_f32<_Float16>(dw);
+        rq += lo_to_f32<_Float16>(qw) + hi_to_f32<_Float16>(qw);
+        rd += d0 + d1;
+        dsum += lo_to_f32<_Float16>(ow) * d0 + hi_to_f32<_Float16>(ow) * d1;
+      }
+    }
+#pragma unroll
+    for (int m = 1; m < 8; m *= 2) {
+      dsum += __shfl_xor(dsum, m, 64);
+      rq += __shfl_xor(rq, m, 64);
+      rd += __shfl_xor(rd, m, 64);
+    }
+    if (part == 0) {
+      const int qi = 32 * qb + pi;
+      stat[pi] = qi < a.Nq ? a.lse[tq0 + qi] * kLog2e : INFINITY;
+      stat[32 + pi] = dsum;
+      stat[64 + pi] = rq;
+      stat[96 + pi] = rd;
+    }
+  };
+  auto load_o = [&](int qb, u32x4 *og) {   // one buffer: this thread's chunks of O straight from memory
+    const int pi = tid / 8, part = tid % 8;
+    const bool live = 32 * qb + pi < a.Nq;
+#pragma unroll
+    for (int k = 0; k < (CPR + 7) / 8; ++k)
+      og[k] = live ? *reinterpret_cast<const u32x4 *>(o_bh + (int64_t)(32 * qb + pi) * a.son + (part + 8 * k) * 8)
+                   : u32x4{0u, 0u, 0u, 0u};
+  };
 
-  // ---- this wave's tile: copy, then its code operands expanded once (B operands: column = key lr)
-  if (t_ok) {
-    Copy cp;
-    cp.init((unsigned)a.scn, lane);
-    skv_issue_tile<S, D>(cp, slot, reinterpret_cast<const unsigned char *>(a.codes + b * a.scb + h * a.sch), a.scale, a.zp,
-                         tk0, t, a.Nk, a.scn, lane);
-  }
-  issue_rows(0);   // together with the tile: one memory latency for both
-  dma_wait();
-  u32x4 cb[KD];
-  float sk = 0.f;
-  u32x4 corr_k = {0u, 0u, 0u, 0u};
-  if (t_ok) {
-    const int k_swz = KSW::swz(lr);
-#pragma unroll
-    for (int jj = 0; jj < D / 32; ++jj) {
-      const u32x4 kw = *reinterpret_cast<const u32x4 *>(slot + lr * D + (((2 * jj + g) ^ k_swz) << 4));
-      cb[2 * jj] = expand_codes(kw[0], kw[1]);
-      cb[2 * jj + 1] = expand_codes(kw[2], kw[3]);
-    }
-    const unsigned *skp = reinterpret_cast<const unsigned *>(slot + SKV_TILE * D);
-    const unsigned skw = skp[lr], zw = skp[SKV_TILE + lr];
-    sk = std::is_same<S, float>::value ? __builtin_bit_cast(float, skw) : lo_to_f32<_Float16>(skw);
-    const unsigned cz = magic_zp_pair(zw, zw);
-    if (g == 0) {
-      corr_k[0] = cz;
-      corr_k[1] = cz & 0xffffu;
-    }
-  } else {
-#pragma unroll
-    for (int m = 0; m < KD; ++m) cb[m] = u32x4{0u, 0u, 0u, 0u};
-  }
-  const float a_sk = key_ok ? a.sm_scale_log2 * sk : 0.f;
-  const float sm_k = key_ok ? a.sm_scale : 0.f;
+  Copy cp;
+  cp.init((unsigned)a.scn, lane);
+  auto issue_tile = [&](int t) {
+    skv_issue_tile<S, D>(cp, slot, codes_bh, a.scale, a.zp, tk0, t, a.Nk, a.scn, lane);
+  };
 
   // ---- per-lane LDS offsets inside a row block (as in the fused kernel)
   const unsigned lds0 = lds_addr(smem);
@@ -374,69 +398,36 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
       qt_off[hh][r] = i * (D * 2) + ((chk ^ RowSwz<D>::swz(i)) << 4) + 8 * (s16 % 2);
     }
 
+  // ---- this wave's tile in registers: code operands (B operands: column = key lr), scale, offset operand
+  u32x4 cb[KD];
+  float sk = 0.f;
+  u32x4 corr_k = {0u, 0u, 0u, 0u};
+  auto expand_tile = [&]() {
+    const int k_swz = KSW::swz(lr);
+#pragma unroll
+    for (int jj = 0; jj < D / 32; ++jj) {
+      const u32x4 kw = *reinterpret_cast<const u32x4 *>(slot + lr * D + (((2 * jj + g) ^ k_swz) << 4));
+      cb[2 * jj] = expand_codes(kw[0], kw[1]);
+      cb[2 * jj + 1] = expand_codes(kw[2], kw[3]);
+    }
+    const unsigned *skp = reinterpret_cast<const unsigned *>(slot + SKV_TILE * D);
+    const unsigned skw = skp[lr], zw = skp[SKV_TILE + lr];
+    sk = std::is_same<S, float>::value ? __builtin_bit_cast(float, skw) : lo_to_f32<_Float16>(skw);
+    const unsigned cz = magic_zp_pair(zw, zw);
+    corr_k = u32x4{0u, 0u, 0u, 0u};
+    if (g == 0) {
+      corr_k[0] = cz;
+      corr_k[1] = cz & 0xffffu;
+    }
+  };
+
   f32x16 dkv[DBW];
-#pragma unroll
-  for (int db = 0; db < DBW; ++db)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) dkv[db][v] = 0.f;
-
-  for (int qb = 0; qb < nqb; ++qb) {
-    unsigned char *buf = smem + (qb % NRB) * SM::BUF;
-    float *stat = reinterpret_cast<float *>(smem + SM::OFF_STAT) + (qb % NRB) * 128;
-    if (NRB == 1 && qb > 0) {
-      __syncthreads();   // everybody is done with block qb-1
-      issue_rows(qb);
-    }
-    // (one buffer: O does not pass through LDS; this thread's chunks of it are fetched while the copy lands)
-    u32x4 og[SM::O_IN_LDS ? 1 : (CPR + 7) / 8];
-    if (!SM::O_IN_LDS) {
-      const int pi = tid / 8, part = tid % 8;
-      const bool live = 32 * qb + pi < a.Nq;
-#pragma unroll
-      for (int k = 0; k < (CPR + 7) / 8; ++k)
-        og[k] = live ? *reinterpret_cast<const u32x4 *>(o_bh + (int64_t)(32 * qb + pi) * a.son + (part + 8 * k) * 8)
-                     : u32x4{0u, 0u, 0u, 0u};
-    }
-    dma_wait();          // this thread's share of block qb has landed ...
-    __syncthreads();     // ... and everybody's; (two buffers:) everybody is also done with block qb-1
-    // ---- delta, row sums, LSE of the block (thread = row tid/8, chunks tid%8 + {0, 8})
-    {
-      const int pi = tid / 8, part = tid % 8;
-      float dsum = 0.f, rq = 0.f, rd = 0.f;
-#pragma unroll
-      for (int c = part; c < CPR; c += 8) {
-        const int off = pi * (D * 2) + ((c ^ RowSwz<D>::swz(pi)) << 4);
-        const u32x4 qv = *reinterpret_cast<const u32x4 *>(buf + off);
-        const u32x4 dv = *reinterpret_cast<const u32x4 *>(buf + SM::ROWS + off);
-        const u32x4 ov = SM::O_IN_LDS ? *reinterpret_cast<const u32x4 *>(buf + 2 * SM::ROWS + off) : og[c / 8];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const unsigned qw = qv[e], dw = dv[e], ow = ov[e];
-          const float d0 = lo_to_f32<_Float16>(dw), d1 = hi_to_f32<_Float16>(dw);
-          rq += lo_to_f32<_Float16>(qw) + hi_to_f32<_Float16>(qw);
-          rd += d0 + d1;
-          dsum += lo_to_f32<_Float16>(ow) * d0 + hi_to_f32<_Float16>(ow) * d1;
-        }
-      }
-#pragma unroll
-      for (int m = 1; m < 8; m *= 2) {
-        dsum += __shfl_xor(dsum, m, 64);
-        rq += __shfl_xor(rq, m, 64);
-        rd += __shfl_xor(rd, m, 64);
-      }
-      if (part == 0) {
-        const int qi = 32 * qb + pi;
-        stat[pi] = qi < a.Nq ? a.lse[tq0 + qi] * kLog2e : INFINITY;
-        stat[32 + pi] = dsum;
-        stat[64 + pi] = rq;
-        stat[96 + pi] = rd;
-      }
-    }
-    if (NRB == 2 && qb + 1 < nqb) issue_rows(qb + 1);   // the other buffer: nobody reads it any more
-    __syncthreads();
-    if (!t_ok) continue;
-
-    // ---- S = Q C^T, dP = dO C^T (rows = queries, columns = keys), rank-1 offset removal
+  // dKV^T of this wave's tile += contributions of query block qb (its rows and statistics are in LDS)
+  auto add_block = [&](int qb, bool key_ok) {
+    const unsigned char *buf = smem + (qb % NRB) * SM::BUF;
+    const float *stat = reinterpret_cast<const float *>(smem + SM::OFF_STAT) + (qb % NRB) * 128;
+    const float a_sk = key_ok ? a.sm_scale_log2 * sk : 0.f;
+    const float sm_k = key_ok ? a.sm_scale : 0.f;
     auto split3 = [&](float rs) -> u32x4 {
       const _Float16 h0 = (_Float16)rs;
       const float r1 = rs - (float)h0;
@@ -449,6 +440,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
       }
       return r;
     };
+    // S = Q C^T, dP = dO C^T (rows = queries, columns = keys), rank-1 offset removal
     f32x16 sacc, pacc;
 #pragma unroll
     for (int v = 0; v < 16; ++v) sacc[v] = 0.f, pacc[v] = 0.f;
@@ -462,7 +454,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
     }
     sacc = mfma_h(split3(stat[64 + lr]), corr_k, sacc);
     pacc = mfma_h(split3(stat[96 + lr]), corr_k, pacc);
-    // ---- p and ds for this lane's key; registers run over the queries 8aa + 4g + bb
+    // p and ds for this lane's key; registers run over the queries 8aa + 4g + bb
     u32x4 pf[2], df[2];
 #pragma unroll
     for (int aa = 0; aa < 4; ++aa) {
@@ -481,7 +473,7 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
         df[aa / 2][2 * (aa % 2) + e] = pack_h2(ds[2 * e], ds[2 * e + 1]);
       }
     }
-    // ---- dKV^T += dO^T P + Q^T dS
+    // dKV^T += dO^T P + Q^T dS
     const unsigned bufa = lds0 + (qb % NRB) * SM::BUF;
 #pragma unroll
     for (int db = 0; db < DBW; ++db) {
@@ -502,12 +494,9 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
         dkv[db] = mfma_h(u32x4{q0[0], q0[1], q1[0], q1[1]}, df[hh], dkv[db]);
       }
     }
-  }
-
-  // ---- the tile's dKV rows leave through an LDS stage as whole 128-byte lines (two 32-column blocks a time)
-  __syncthreads();   // the row buffers are done with: the stages overlay them
-  if (t_ok) {
-    unsigned char *stage = smem + wave * SM::STAGE;   // (row buffers)
+  };
+  // the tile's dKV rows leave through a 4 KB LDS stage as whole 128-byte lines (two 32-column blocks a time)
+  auto write_out = [&](unsigned char *stage, int j0) {
     _Float16 *dkv_bh = a.dkv + b * a.sdkb + h * a.sdkh;
     const int st_w = lr * 128 + 8 * g, st_wswz = lr % 8;
     const int st_r = (lane / 8) * 128 + (((lane % 8) ^ (lane / 8)) << 4);
@@ -529,7 +518,81 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dkv_k
         }
       }
     }
+  };
+  auto clear_dkv = [&]() {
+#pragma unroll
+    for (int db = 0; db < DBW; ++db)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) dkv[db][v] = 0.f;
+  };
+
+  if (KEEP) {
+    // ---- rows of every query block and the first tile, copied together; statistics once
+    if (tile_of(c_begin) < ntiles) issue_tile(tile_of(c_begin));
+    for (int qb = 0; qb < nqb; ++qb) issue_rows(qb);
+    u32x4 og[SM::O_IN_LDS ? 1 : (CPR + 7) / 8];
+    if (!SM::O_IN_LDS) load_o(0, og);
+    dma_wait();
+    __syncthreads();
+    for (int qb = 0; qb < nqb; ++qb) block_stats(qb, og);
+    __syncthreads();
+    // stage: in the O rows (waves 0,1 use buffer 0's, waves 2,3 buffer 1's), in an area of its own, or in the
+    // wave's tile slot once its operands are in registers
+    unsigned char *stage = SM::STAGE_MODE == 0 ? smem + (wave / 2) * SM::BUF + 2 * SM::ROWS + (wave % 2) * SM::STAGE
+                           : SM::STAGE_MODE == 1 ? smem + SM::OFF_STAGE + wave * SM::STAGE : slot;
+    // The dKV stores share the memory counter with the tile copies, so the wait for the next tile sits
+    // BEFORE the stores of the current one: by then the copy, issued a whole compute phase earlier, is the
+    // only thing that can still be in flight.  (Stage in the slot: the copy can only be issued after the
+    // stores, and the wait at the top of the next round also covers them.)
+    for (int c = c_begin; c < c_end; ++c) {
+      const int t = tile_of(c);
+      if (t >= ntiles) break;   // (tiles of a wave grow with c)
+      if (SM::STAGE_MODE == 2) dma_wait();
+      expand_tile();
+      const int tn = tile_of(c + 1);
+      const bool more = c + 1 < c_end && tn < ntiles;
+      if (SM::STAGE_MODE != 2 && more) {   // the slot is free once its contents are in registers
+        lds_wait_all();
+        issue_tile(tn);
+      }
+      clear_dkv();
+      const int j0 = t * SKV_TILE;
+      for (int qb = 0; qb < nqb; ++qb) add_block(qb, j0 + lr < a.Nk);
+      if (SM::STAGE_MODE != 2) dma_wait();
+      write_out(stage, j0);
+      if (SM::STAGE_MODE == 2 && more) {   // the stage was the slot: refill it only now
+        lds_wait_all();
+        issue_tile(tn);
+      }
+    }
+    return;
   }
+
+  // ---- one chunk per workgroup, the row blocks cycle through the buffers
+  const int t = tile_of(c_begin);
+  const bool t_ok = t < ntiles;                   // (a wave without a tile still takes part in copies and barriers)
+  const int j0 = t * SKV_TILE;
+  if (t_ok) issue_tile(t);
+  issue_rows(0);   // together with the tile: one memory latency for both
+  dma_wait();
+  if (t_ok) expand_tile();
+  clear_dkv();
+  for (int qb = 0; qb < nqb; ++qb) {
+    if (NRB == 1 && qb > 0) {
+      __syncthreads();   // everybody is done with block qb-1
+      issue_rows(qb);
+    }
+    u32x4 og[SM::O_IN_LDS ? 1 : (CPR + 7) / 8];
+    if (!SM::O_IN_LDS) load_o(qb, og);
+    dma_wait();          // this thread's share of block qb has landed ...
+    __syncthreads();     // ... and everybody's; (two buffers:) everybody is also done with block qb-1
+    block_stats(qb, og);
+    if (NRB == 2 && qb + 1 < nqb) issue_rows(qb + 1);   // the other buffer: nobody reads it any more
+    __syncthreads();
+    if (t_ok) add_block(qb, j0 + lr < a.Nk);
+  }
+  __syncthreads();   // the row buffers are done with: the stages overlay them
+  if (t_ok) write_out(smem + wave * SM::STAGE, j0);
 }
 
 template <typename S, int D> static int launch_skv_bwd_long_sd(const SkvAttnArgs &x, hipStream_t st) {
@@ -549,12 +612,22 @@ template <typename S, int D> static int launch_skv_bwd_long_sd(const SkvAttnArgs
   a.qblocks = (int)((x.Nq + 15) / 16);
   const int keys_per_wg = 4 * SKV_TILE / SkvDkvSmem<D>::DS;
   a.kchunks = (int)((x.Nk + keys_per_wg - 1) / keys_per_wg);
-  const int64_t total_q = (int64_t)a.qblocks * ((a.BH + 7) / 8) * 8, total_k = (int64_t)a.kchunks * a.BH;
+  // query blocks that fit the row buffers stay resident and a workgroup walks over several chunks: as many
+  // as leave about 2048 workgroups (four rounds of two per CU)
+  const bool keep = x.Nq <= 32 * SkvDkvSmem<D>::NRB;
+  a.cpw = 1;
+  if (keep) {
+    const int64_t want = ((int64_t)a.kchunks * a.BH + 2047) / 2048;
+    a.cpw = (int)(want < 1 ? 1 : want > a.kchunks ? a.kchunks : want);
+  }
+  const int64_t total_q = (int64_t)a.qblocks * ((a.BH + 7) / 8) * 8;
+  const int64_t total_k = (int64_t)((a.kchunks + a.cpw - 1) / a.cpw) * a.BH;
   if (total_q > 0x7fffffffLL || total_k > 0x7fffffffLL)
     return set_error(QFA_EUNSUPPORTED, "attn_bwd_shared_kv: too many blocks for one launch");
   skv_dq_kernel<S, D><<<dim3((unsigned)total_q), dim3(256), 0, st>>>(a);
   if (int e = check_launch("qfa_attn_bwd_shared_kv (dQ)")) return e;
-  skv_dkv_kernel<S, D><<<dim3((unsigned)total_k), dim3(256), 0, st>>>(a);
+  if (keep) skv_dkv_kernel<S, D, true><<<dim3((unsigned)total_k), dim3(256), 0, st>>>(a);
+  else skv_dkv_kernel<S, D, false><<<dim3((unsigned)total_k), dim3(256), 0, st>>>(a);
   return check_launch("qfa_attn_bwd_shared_kv (dKV)");
 }
 
