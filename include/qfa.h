@@ -131,12 +131,17 @@ int qfa_attn_fwd_shared_kv(const void *q, const int8_t *codes, const void *scale
  * (batch, head) run in one fused pass (one workgroup per (batch, head) streams the codes once and
  * writes each dKV row once); longer query blocks run a dQ kernel (one workgroup per 16 queries) and
  * a dKV kernel (one workgroup per 128 keys walking over the queries).
- *   q, o, dout, dq [B,H,Nq,D] and dkv [B,H,Nk,D] fp16 (io_dtype must be QFA_F16), strides as given;
+ *   q, o, dout [B,H,Nq,D] fp16 (io_dtype must be QFA_F16: the kernels compute in binary16), strides as given;
+ *   dq [B,H,Nq,D], dkv [B,H,Nk,D] of grad_dtype (QFA_F16 or QFA_BF16);
+ *   grad_scale  nullable DEVICE pointer to one float that multiplies dq and dkv before they are rounded.
+ *               dQ and dKV are linear in dO: a caller whose dO does not fit binary16 (bf16 training) hands
+ *               over dO * 2^k and *grad_scale = 2^-k without a host synchronisation;
  *   codes, scale, scale_dtype, zp, lse as in the forward.  D in {64, 128, 256} (256: always the two kernels).
  *   The sums of a query's and of a dO row's D elements must stay inside binary16 range.
  */
 int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp,
                            const void *o, const void *dout, const float *lse, void *dq, void *dkv, int io_dtype,
+                           int grad_dtype, const float *grad_scale,
                            int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D, int64_t sqb, int64_t sqh, int64_t sqn,
                            int64_t scb, int64_t sch, int64_t scn, int64_t sob, int64_t soh, int64_t son, int64_t sdob,
                            int64_t sdoh, int64_t sdon, int64_t sdqb, int64_t sdqh, int64_t sdqn, int64_t sdkb,

@@ -170,6 +170,7 @@ int qfa_attn_fwd_shared_kv(const void *q, const int8_t *codes, const void *scale
 
 int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp,
                            const void *o, const void *dout, const float *lse, void *dq, void *dkv, int io_dtype,
+                           int grad_dtype, const float *grad_scale,
                            int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D, int64_t sqb, int64_t sqh, int64_t sqn,
                            int64_t scb, int64_t sch, int64_t scn, int64_t sob, int64_t soh, int64_t son, int64_t sdob,
                            int64_t sdoh, int64_t sdon, int64_t sdqb, int64_t sdqh, int64_t sdqn, int64_t sdkb,
@@ -178,7 +179,7 @@ int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale
   SkvAttnArgs a;
   memset(&a, 0, sizeof(a));
   a.q = q; a.codes = codes; a.scale = scale; a.zp = zp; a.o = const_cast<void *>(o); a.lse = const_cast<float *>(lse);
-  a.dout = dout; a.dq = dq; a.dkv = dkv;
+  a.dout = dout; a.dq = dq; a.dkv = dkv; a.grad_dtype = grad_dtype; a.grad_scale = grad_scale;
   a.B = B; a.H = H; a.Nq = Nq; a.Nk = Nk; a.D = D; a.io_dtype = io_dtype; a.scale_dtype = scale_dtype;
   a.sqb = sqb; a.sqh = sqh; a.sqn = sqn; a.scb = scb; a.sch = sch; a.scn = scn; a.sob = sob; a.soh = soh; a.son = son;
   a.sdob = sdob; a.sdoh = sdoh; a.sdon = sdon; a.sdqb = sdqb; a.sdqh = sdqh; a.sdqn = sdqn;
@@ -186,7 +187,9 @@ int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale
   a.sm_scale = sm_scale;
   if (int e = check_shared_kv(who, a)) return e;
   if (!dout || !dq || !dkv) return set_error(QFA_EINVAL, "%s: null pointer argument", who);
-  if (io_dtype != QFA_F16) return set_error(QFA_EUNSUPPORTED, "%s: io_dtype must be QFA_F16", who);
+  if (io_dtype != QFA_F16) return set_error(QFA_EUNSUPPORTED, "%s: io_dtype (q, o, dout) must be QFA_F16", who);
+  if (grad_dtype != QFA_F16 && grad_dtype != QFA_BF16)
+    return set_error(QFA_EINVAL, "%s: grad_dtype (dq, dkv) must be QFA_F16 or QFA_BF16", who);
   if (!aligned16(dout) || !aligned16(dq) || !aligned16(dkv))
     return set_error(QFA_EINVAL, "%s: dout, dq, dkv must be 16-byte aligned", who);
   if (!strides_ok(sdob, sdoh, sdon, D, 2) || !strides_ok(sdqb, sdqh, sdqn, D, 2) || !strides_ok(sdkb, sdkh, sdkn, D, 2))

@@ -52,6 +52,7 @@ struct SkvAttnArgs {
   int64_t sdob, sdoh, sdon, sdqb, sdqh, sdqn, sdkb, sdkh, sdkn;
   float sm_scale;
   int D, io_dtype, scale_dtype;
+  int grad_dtype; const float *grad_scale;   // backward only: type of dq / dkv, optional device scalar multiplying them
 };
 int launch_skv_fwd(const SkvAttnArgs &a, hipStream_t st);
 int64_t skv_fwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D);

@@ -34,7 +34,9 @@ struct SkvBwdArgs {
   const _Float16 *q, *o, *dout;
   const int8_t *codes; const void *scale; const int8_t *zp;
   const float *lse;
-  _Float16 *dq, *dkv;
+  _Float16 *dq, *dkv;          // 16-bit outputs: binary16, or bfloat16 when grad_bf16 is set
+  const float *grad_scale;     // nullable device scalar: dq and dkv are multiplied by it before rounding
+  int grad_bf16;
   int64_t H;
   int Nq, Nk;
   int64_t sqb, sqh, sqn, scb, sch, scn, sob, soh, son, sdob, sdoh, sdon, sdqb, sdqh, sdqn, sdkb, sdkh, sdkn;
@@ -86,6 +88,10 @@ template <typename S, int D, bool HALF> __global__ __launch_bounds__(256, 2) voi
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int wave_off = wave * SM::WAVE;
   float *stat = reinterpret_cast<float *>(smem + SM::OFF_STAT);
+  const float osc = a.grad_scale ? *a.grad_scale : 1.0f;
+  auto pack_out = [&](float x, float y) -> unsigned {
+    return a.grad_bf16 ? pack2<__bf16>(x * osc, y * osc) : pack2<_Float16>(x * osc, y * osc);
+  };
 
   const unsigned char *codes_bh = reinterpret_cast<const unsigned char *>(a.codes + b * a.scb + h * a.sch);
   const int64_t tk0 = (int64_t)bh * a.Nk, tq0 = (int64_t)bh * a.Nq;
@@ -350,8 +356,8 @@ template <typename S, int D, bool HALF> __global__ __launch_bounds__(256, 2) voi
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa) {
         u32x2 o2;
-        o2[0] = pack_h2(acc[4 * aa], acc[4 * aa + 1]);
-        o2[1] = pack_h2(acc[4 * aa + 2], acc[4 * aa + 3]);
+        o2[0] = pack_out(acc[4 * aa], acc[4 * aa + 1]);
+        o2[1] = pack_out(acc[4 * aa + 2], acc[4 * aa + 3]);
         *reinterpret_cast<u32x2 *>(stage + st_w + (((4 * (db % 2) + aa) ^ st_wswz) << 4)) = o2;
       }
       if (db % 2 == 1) {
@@ -404,8 +410,8 @@ template <typename S, int D, bool HALF> __global__ __launch_bounds__(256, 2) voi
           r[bb] = dq[db][4 * aa + bb] - w_tot + mg[d * 32 + lr] + mg[MG + d * 32 + lr] + mg[2 * MG + d * 32 + lr];
         }
         u32x2 o2;
-        o2[0] = pack_h2(r[0], r[1]);
-        o2[1] = pack_h2(r[2], r[3]);
+        o2[0] = pack_out(r[0], r[1]);
+        o2[1] = pack_out(r[2], r[3]);
         *reinterpret_cast<u32x2 *>(qrow + 32 * db + 8 * aa + 4 * g) = o2;
       }
   }
@@ -417,6 +423,7 @@ template <typename S, int D> static int launch_skv_bwd_sd(const SkvAttnArgs &x, 
   a.dout = static_cast<const _Float16 *>(x.dout);
   a.codes = x.codes; a.scale = x.scale; a.zp = x.zp; a.lse = x.lse;
   a.dq = static_cast<_Float16 *>(x.dq); a.dkv = static_cast<_Float16 *>(x.dkv);
+  a.grad_scale = x.grad_scale; a.grad_bf16 = x.grad_dtype == QFA_BF16;
   a.H = x.H; a.Nq = (int)x.Nq; a.Nk = (int)x.Nk;
   a.sqb = x.sqb; a.sqh = x.sqh; a.sqn = x.sqn; a.scb = x.scb; a.sch = x.sch; a.scn = x.scn;
   a.sob = x.sob; a.soh = x.soh; a.son = x.son; a.sdob = x.sdob; a.sdoh = x.sdoh; a.sdon = x.sdon;

@@ -28,7 +28,9 @@ struct SkvBwdLongArgs {
   const _Float16 *q, *o, *dout;
   const int8_t *codes; const void *scale; const int8_t *zp;
   const float *lse;
-  _Float16 *dq, *dkv;
+  _Float16 *dq, *dkv;          // 16-bit outputs: binary16, or bfloat16 when grad_bf16 is set
+  const float *grad_scale;     // nullable device scalar: dq and dkv are multiplied by it before rounding
+  int grad_bf16;
   int64_t H;
   int Nq, Nk, BH, qblocks, kchunks, cpw;   // cpw: key chunks per workgroup of the dKV kernel
   int64_t sqb, sqh, sqn, scb, sch, scn, sob, soh, son, sdob, sdoh, sdon, sdqb, sdqh, sdqn, sdkb, sdkh, sdkn;
@@ -68,6 +70,10 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dq_ke
   };
   auto scale_of = [](unsigned w) -> float {
     return std::is_same<S, float>::value ? __builtin_bit_cast(float, w) : lo_to_f32<_Float16>(w);
+  };
+  const float osc = a.grad_scale ? *a.grad_scale : 1.0f;
+  auto pack_out = [&](float x, float y) -> unsigned {
+    return a.grad_bf16 ? pack2<__bf16>(x * osc, y * osc) : pack2<_Float16>(x * osc, y * osc);
   };
 #pragma unroll
   for (int i = 0; i < SKVQ_NBUF - 1; ++i)
@@ -250,8 +256,8 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dq_ke
         r[v] = acc[db][v] - w_tot + mg[d * 16 + q16] + mg[MG + d * 16 + q16] + mg[2 * MG + d * 16 + q16];
       }
       u32x2 o2;
-      o2[0] = pack_h2(r[0], r[1]);
-      o2[1] = pack_h2(r[2], r[3]);
+      o2[0] = pack_out(r[0], r[1]);
+      o2[1] = pack_out(r[2], r[3]);
       *reinterpret_cast<u32x2 *>(out + 16 * db + 4 * G) = o2;
     }
   }
@@ -312,6 +318,10 @@ template <typename S, int D, bool KEEP> __global__ __launch_bounds__(256, 2) voi
   const int64_t tk0 = (int64_t)bh * a.Nk, tq0 = (int64_t)bh * a.Nq;
   const int nqb = (a.Nq + 31) / 32;
   auto tile_of = [&](int chunk) { return (4 / DS) * chunk + wave / DS; };   // this wave's tile in a chunk
+  const float osc = a.grad_scale ? *a.grad_scale : 1.0f;
+  auto pack_out = [&](float x, float y) -> unsigned {
+    return a.grad_bf16 ? pack2<__bf16>(x * osc, y * osc) : pack2<_Float16>(x * osc, y * osc);
+  };
 
   // ---- row copies of a query block: Q, dO (, O) -> buffer (direct loads)
   RowCopy cq, cd, co;
@@ -505,8 +515,8 @@ template <typename S, int D, bool KEEP> __global__ __launch_bounds__(256, 2) voi
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa) {
         u32x2 o2;
-        o2[0] = pack_h2(dkv[db][4 * aa], dkv[db][4 * aa + 1]);
-        o2[1] = pack_h2(dkv[db][4 * aa + 2], dkv[db][4 * aa + 3]);
+        o2[0] = pack_out(dkv[db][4 * aa], dkv[db][4 * aa + 1]);
+        o2[1] = pack_out(dkv[db][4 * aa + 2], dkv[db][4 * aa + 3]);
         *reinterpret_cast<u32x2 *>(stage + st_w + (((4 * (db % 2) + aa) ^ st_wswz) << 4)) = o2;
       }
       if (db % 2 == 1) {
@@ -601,6 +611,7 @@ template <typename S, int D> static int launch_skv_bwd_long_sd(const SkvAttnArgs
   a.dout = static_cast<const _Float16 *>(x.dout);
   a.codes = x.codes; a.scale = x.scale; a.zp = x.zp; a.lse = x.lse;
   a.dq = static_cast<_Float16 *>(x.dq); a.dkv = static_cast<_Float16 *>(x.dkv);
+  a.grad_scale = x.grad_scale; a.grad_bf16 = x.grad_dtype == QFA_BF16;
   a.H = x.H; a.Nq = (int)x.Nq; a.Nk = (int)x.Nk;
   a.sqb = x.sqb; a.sqh = x.sqh; a.sqn = x.sqn; a.scb = x.scb; a.sch = x.sch; a.scn = x.scn;
   a.sob = x.sob; a.soh = x.soh; a.son = x.son; a.sdob = x.sdob; a.sdoh = x.sdoh; a.sdon = x.sdon;

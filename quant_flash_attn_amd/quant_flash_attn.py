@@ -11,8 +11,9 @@ Two autograd entry points, both backed by the HIP kernels behind qfa_attn_fwd / 
       The reference's own entry point (quant_flash_attn.py:173-240): one quantized tensor serves as
       K and V, `kv_fp16` only receives the gradient, backward returns (dq, dkv, None, None) with
       dkv = dK + dV (:161).  Query blocks of up to SHARED_KV_MAX_Q (512) tokens run the reference's
-      computation itself in the forward (Q in 16-bit, qfa_attn_fwd_shared_kv), and in fp16 also in
-      the backward (qfa_attn_bwd_shared_kv).  Everything else goes through the INT8-score kernels, where Q is quantized per token too (stated
+      computation itself in the forward (Q in 16-bit, qfa_attn_fwd_shared_kv) and in the backward
+      (qfa_attn_bwd_shared_kv, binary16 arithmetic; bf16 tensors are converted around it).  Longer
+      query blocks go through the INT8-score kernels, where Q is quantized per token too (stated
       difference from the reference, which keeps Q in fp16).
 """
 from __future__ import annotations
@@ -163,14 +164,20 @@ def attn_fwd_shared_kv(q: torch.Tensor, codes: torch.Tensor, scale: torch.Tensor
 
 
 def attn_bwd_shared_kv(q: torch.Tensor, codes: torch.Tensor, scale: torch.Tensor, zero_point: torch.Tensor,
-                       o: torch.Tensor, do: torch.Tensor, lse: torch.Tensor, sm_scale: float
+                       o: torch.Tensor, do: torch.Tensor, lse: torch.Tensor, sm_scale: float,
+                       grad_dtype: Optional[torch.dtype] = None, grad_scale: Optional[torch.Tensor] = None
                        ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """dQ, dKV of attn_fwd_shared_kv in fp16: the computation of _attn_bwd_kernel_quantized
+    """dQ, dKV of attn_fwd_shared_kv: the computation of _attn_bwd_kernel_quantized
     (quant_flash_attn.py:104-166) with dKV = dV + dK as stored there (:161).  q, o, do fp16
-    [B,H,Nq,D]; lse as returned by the forward.  Up to 32 queries run in one fused pass over the codes,
-    longer blocks in a dQ kernel plus a dKV kernel."""
+    [B,H,Nq,D] (the kernels compute in binary16); lse as returned by the forward.  dQ and dKV come back
+    in `grad_dtype` (fp16 by default, or bf16), multiplied by the one-element device tensor `grad_scale`
+    if given.  Up to 32 queries run in one fused pass over the codes, longer blocks (and head_dim 256)
+    in a dQ kernel plus a dKV kernel."""
     if q.dtype != torch.float16 or o.dtype != torch.float16:
         raise TypeError("the shared-KV backward kernel computes in float16: q and o must be float16")
+    grad_dtype = grad_dtype or torch.float16
+    if grad_dtype not in _IO_DTYPES:
+        raise TypeError(f"grad_dtype must be float16 or bfloat16, got {grad_dtype}")
     if codes.dim() != 4 or codes.dtype != torch.int8:
         raise ValueError("codes must be a 4-D int8 tensor")
     B, H, Nq, D = q.shape
@@ -179,6 +186,9 @@ def attn_bwd_shared_kv(q: torch.Tensor, codes: torch.Tensor, scale: torch.Tensor
         raise ValueError("shape mismatch between q / o / do and the codes")
     do = do.to(torch.float16)
     _lib.require_gpu(q, codes, scale, zero_point, o, do, lse)
+    if grad_scale is not None:
+        _lib.require_gpu(q, grad_scale)
+        grad_scale = _flat(grad_scale, torch.float32, 1, "grad_scale")
     n = B * H * Nk
     if scale.dtype not in (torch.float32, torch.float16):
         scale = scale.to(torch.float32)
@@ -186,13 +196,14 @@ def attn_bwd_shared_kv(q: torch.Tensor, codes: torch.Tensor, scale: torch.Tensor
     zero_point = _flat(zero_point, torch.int8, n, "zero_point")
     lse = _flat(lse, torch.float32, B * H * Nq, "lse")
     q, codes, o, do = _rows16(q), _rows16(codes), _rows16(o), _rows16(do)
-    dq = torch.empty((B, H, Nq, D), dtype=torch.float16, device=q.device)
-    dkv = torch.empty((B, H, Nk, D), dtype=torch.float16, device=q.device)
+    dq = torch.empty((B, H, Nq, D), dtype=grad_dtype, device=q.device)
+    dkv = torch.empty((B, H, Nk, D), dtype=grad_dtype, device=q.device)
     s = lambda t: (t.stride(0), t.stride(1), t.stride(2))
     with torch.cuda.device(q.device):
         code = _lib.lib().qfa_attn_bwd_shared_kv(
             q.data_ptr(), codes.data_ptr(), scale.data_ptr(), _lib.DTYPE_CODE[scale.dtype], zero_point.data_ptr(),
             o.data_ptr(), do.data_ptr(), lse.data_ptr(), dq.data_ptr(), dkv.data_ptr(), _lib.QFA_F16,
+            _lib.DTYPE_CODE[grad_dtype], grad_scale.data_ptr() if grad_scale is not None else None,
             B, H, Nq, Nk, D, *s(q), *s(codes), *s(o), *s(do), *s(dq), *s(dkv), float(sm_scale), _lib.stream_of(q))
     _lib.check(code, "qfa_attn_bwd_shared_kv")
     return dq, dkv
@@ -272,7 +283,16 @@ class QuantFlashAttention(torch.autograd.Function):
             if q.dtype == torch.float16:
                 dq, dkv = attn_bwd_shared_kv(q, codes, scale, zp, o, grad_output, lse, ctx.sm_scale)
                 return dq, dkv.to(ctx.kv_dtype), None, None
-            qq, kq, v16 = _legacy_operands(q, codes, scale, zp, q.dtype)
+            # bf16: the backward kernels compute in binary16.  q and o convert exactly (more mantissa, values
+            # of order one); dO may lie below binary16's range, so it is handed over scaled by a power of two
+            # chosen on the device from its largest magnitude (no synchronisation), and the kernels scale dQ
+            # and dKV -- linear in dO -- back while they round them to bf16.
+            do32 = grad_output.to(torch.float32)
+            k = torch.floor(torch.log2(256.0 / do32.abs().amax().clamp_min(1e-30))).clamp_(-100.0, 100.0)
+            dq, dkv = attn_bwd_shared_kv(q.to(torch.float16), codes, scale, zp, o.to(torch.float16),
+                                         (do32 * torch.exp2(k)).to(torch.float16), lse, ctx.sm_scale,
+                                         grad_dtype=torch.bfloat16, grad_scale=torch.exp2(-k))
+            return dq.to(ctx.q_dtype), dkv.to(ctx.kv_dtype), None, None
         else:
             qq, kq = QuantizedTokens(*t[0:4]), QuantizedTokens(*t[4:8])
             v16, o, lse = t[8], t[9], t[10]

@@ -70,13 +70,14 @@ def test_argument_errors_need_no_gpu(qfa):
     assert skv_fwd(io=0) == -1 and b"io_dtype" in L.qfa_last_error()
     assert skv_fwd(io=1, sdt=2) == -1 and b"scale_dtype" in L.qfa_last_error()
     assert skv_fwd(sm=float("nan")) == -1 and b"sm_scale" in L.qfa_last_error()
-    def skv_bwd(Nq=16, Nk=100, D=128, io=1, dkv=ok_ptr):
+    def skv_bwd(Nq=16, Nk=100, D=128, io=1, dkv=ok_ptr, gd=1):
         sq, sc = (Nq * D, Nq * D, D), (Nk * D, Nk * D, D)
         return L.qfa_attn_bwd_shared_kv(ok_ptr, ok_ptr, ok_ptr, 0, ok_ptr, ok_ptr, ok_ptr, ok_ptr, ok_ptr, dkv, io,
-                                        1, 1, Nq, Nk, D, *sq, *sc, *sq, *sq, *sq, *sc, 0.1, None)
+                                        gd, None, 1, 1, Nq, Nk, D, *sq, *sc, *sq, *sq, *sq, *sc, 0.1, None)
     assert skv_bwd(D=96) == -2 and b"head_dim" in L.qfa_last_error()
     assert skv_bwd(io=2) == -2 and b"QFA_F16" in L.qfa_last_error()
     assert skv_bwd(dkv=None) == -1 and b"null" in L.qfa_last_error()
+    assert skv_bwd(gd=0) == -1 and b"grad_dtype" in L.qfa_last_error()
 
 
 def test_cpu_tensors_are_refused_not_emulated(qfa):

@@ -117,6 +117,30 @@ def test_shared_kv_entry_point_autograd(qfa):
     assert kvd.grad.dtype == torch.float16 and qd.grad.dtype == torch.float16
 
 
+@pytest.mark.parametrize("do_scale", [1.0, 2.0 ** -22])
+def test_shared_kv_entry_point_bf16(qfa, do_scale):
+    """bf16 tensors through the reference's entry point: forward in the shared-KV kernel (queries rounded to
+    binary16), backward in the binary16 kernels with dO scaled into range by a power of two -- also when
+    dO is far below binary16's smallest normal number."""
+    B, H, Nq, Nk, D = 2, 3, 16, 700, 128
+    q, kv = _inputs("normal", B, H, Nq, Nk, D, torch.bfloat16, seed=31)
+    sm = 1.0 / math.sqrt(D)
+    qd = q.to(DEV).requires_grad_(True)
+    kvd = kv.to(DEV).requires_grad_(True)
+    kv_quant = qfa.asymmetric_quant_per_token(kvd.detach())
+    o = qfa.quant_flash_attn(qd, kvd, kv_quant, sm)
+    do = (torch.randn(o.shape, generator=torch.Generator().manual_seed(6)) * do_scale).to(torch.bfloat16)
+    o.backward(do.to(DEV))
+    assert o.dtype == torch.bfloat16 and qd.grad.dtype == torch.bfloat16 and kvd.grad.dtype == torch.bfloat16
+    codes, scale, zp = (t.cpu() for t in kv_quant)
+    o_ref, _ = oracle.legacy_fwd(q, codes, scale, zp, sm)
+    dq_ref, dkv_ref = oracle.legacy_bwd(q, codes, scale, zp, do, sm)
+    assert_close("O", o.detach().cpu(), o_ref, scaled=True)
+    # gradients compared in units of dO's scale (the absolute bound of the contract assumes dO of order one)
+    assert_close("dQ", qd.grad.cpu().double() / do_scale, dq_ref / do_scale, scaled=True)
+    assert_close("dKV", kvd.grad.cpu().double() / do_scale, dkv_ref / do_scale, scaled=True)
+
+
 def test_shared_kv_entry_point_long_query_block(qfa):
     """97 queries (a reference test shape, test_accuracy.py:44): the forward splits them over workgroups
     of 16, the backward runs its dQ and dKV kernels."""
@@ -315,7 +339,7 @@ def test_shared_kv_backward_strided_views(qfa, Nq):
     s3 = lambda t: (t.stride(0), t.stride(1), t.stride(2))
     rc = _lib.lib().qfa_attn_bwd_shared_kv(
         q_v.data_ptr(), c_v.data_ptr(), scale.data_ptr(), _lib.QFA_F16, zp.data_ptr(), o_v.data_ptr(), do_v.data_ptr(),
-        lse.data_ptr(), dq_v.data_ptr(), dkv_v.data_ptr(), _lib.QFA_F16, B, H, Nq, Nk, D,
+        lse.data_ptr(), dq_v.data_ptr(), dkv_v.data_ptr(), _lib.QFA_F16, _lib.QFA_F16, None, B, H, Nq, Nk, D,
         *s3(q_v), *s3(c_v), *s3(o_v), *s3(do_v), *s3(dq_v), *s3(dkv_v), sm, _lib.stream_of(qd))
     assert rc == 0, _lib.lib().qfa_last_error()
     torch.cuda.synchronize()
