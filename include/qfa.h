@@ -106,7 +106,9 @@ int qfa_attn_fwd(const int8_t *qc, const float *sq, const int8_t *zq, const int3
  *   codes  int8 [B,H,Nk,D], strides sc?;  zp int8 [B*H*Nk]
  *   scale  [B*H*Nk] of scale_dtype: QFA_F32, or the same 16-bit type as io_dtype
  *   D in {64, 128, 256}.  q, codes, o 16-byte aligned, strides multiples of 16 bytes, scn < 2^23.
- *   The sum of a query's D elements must stay inside binary16 range (|sum| < 65504).
+ *   The codes' binary16 offset (1152) is removed through the sum of a query's D elements: |sum| must
+ *   stay below 2^21, and the scores carry an absolute error of a few fp32 ulp of 1152 * |sum| code
+ *   units (nothing for |q| of order 10; about a percent of a score once every element is near 500).
  *   workspace  nullable.  With few (batch, head) pairs one workgroup per 16 queries leaves most of the
  *              chip idle (the reference launches one program per (batch, head)); given a caller-owned
  *              scratch of qfa_attn_fwd_shared_kv_workspace_bytes(...) bytes (16-byte aligned; the

@@ -125,16 +125,12 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
   }
   rs += __shfl_xor(rs, 16, 64);
   rs += __shfl_xor(rs, 32, 64);
+  const bool big = offset_needs_x32(rs);
   u32x4 corr_q = {0u, 0u, 0u, 0u};
-  {
-    const _Float16 h0 = (_Float16)rs;
-    const float r1 = rs - (float)h0;
-    const _Float16 h1 = (_Float16)r1;
-    const _Float16 h2 = (_Float16)(r1 - (float)h1);
-    if (G == 0) {
-      corr_q[0] = pack_h2(-(float)h0, -(float)h1);
-      corr_q[1] = pack_h2(-(float)h2, 0.f);
-    }
+  if (G == 0) {
+    const u32x2 cq2 = offset_query_operand(rs, big);
+    corr_q[0] = cq2[0];
+    corr_q[1] = cq2[1];
   }
   const float a_s = a.sm_scale_log2;
 
@@ -187,11 +183,11 @@ template <typename T, typename S, int D> __global__ __launch_bounds__(256, 2) vo
 #pragma unroll
       for (int m = 0; m < KS; ++m)
         f[rb] = mfma_h16(expand_codes(kw[m / 2][2 * (m % 2)], kw[m / 2][2 * (m % 2) + 1]), qf[m], f[rb]);
-      const unsigned cz = magic_zp_pair(z_a[rb], z_a[rb]);
       u32x4 corr_k = {0u, 0u, 0u, 0u};
       if (G == 0) {
-        corr_k[0] = cz;
-        corr_k[1] = cz & 0xffffu;
+        const u32x2 ck2 = offset_key_operand(z_a[rb], big);
+        corr_k[0] = ck2[0];
+        corr_k[1] = ck2[1];
       }
       f[rb] = mfma_h16(corr_k, corr_q, f[rb]);
     }

@@ -169,20 +169,17 @@ template <typename S, int D, bool HALF> __global__ __launch_bounds__(256, 2) voi
   }
   __syncthreads();
 
-  // -rowsum as three binary16 terms in k-group 0: A operand of the rank-1 updates (row = query lr)
-  auto split3 = [&](float rs) -> u32x4 {
-    const _Float16 h0 = (_Float16)rs;
-    const float r1 = rs - (float)h0;
-    const _Float16 h1 = (_Float16)r1;
-    const _Float16 h2 = (_Float16)(r1 - (float)h1);
-    u32x4 r = {0u, 0u, 0u, 0u};
-    if (g == 0) {
-      r[0] = pack_h2(-(float)h0, -(float)h1);
-      r[1] = pack_h2(-(float)h2, 0.f);
-    }
-    return r;
-  };
-  const u32x4 corr_q = split3(stat[64 + lr]), corr_do = split3(stat[96 + lr]);
+  // query-side operands of the rank-1 updates (A operand: row = query lr), one scaling for the whole block
+  const float rs_q = stat[64 + lr], rs_do = stat[96 + lr];
+  const bool big = offset_needs_x32(fmaxf(fabsf(rs_q), fabsf(rs_do)));
+  u32x4 corr_q = {0u, 0u, 0u, 0u}, corr_do = {0u, 0u, 0u, 0u};
+  if (g == 0) {
+    const u32x2 cq2 = offset_query_operand(rs_q, big), cd2 = offset_query_operand(rs_do, big);
+    corr_q[0] = cq2[0];
+    corr_q[1] = cq2[1];
+    corr_do[0] = cd2[0];
+    corr_do[1] = cd2[1];
+  }
   const float a_s = a.sm_scale_log2;
 
   // ---- per-lane LDS offsets
@@ -261,11 +258,11 @@ template <typename S, int D, bool HALF> __global__ __launch_bounds__(256, 2) voi
       }
     }
     {
-      const unsigned cz = magic_zp_pair(zmine, zmine);
       u32x4 corr_k = {0u, 0u, 0u, 0u};
       if (g == 0) {
-        corr_k[0] = cz;
-        corr_k[1] = cz & 0xffffu;
+        const u32x2 ck2 = offset_key_operand(zmine, big);
+        corr_k[0] = ck2[0];
+        corr_k[1] = ck2[1];
       }
       sacc = mfma_h(corr_q, corr_k, sacc);
       pacc = mfma_h(corr_do, corr_k, pacc);

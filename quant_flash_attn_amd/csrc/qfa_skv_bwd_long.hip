@@ -110,19 +110,15 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dq_ke
     rd += __shfl_xor(rd, m, 64);
     delta += __shfl_xor(delta, m, 64);
   }
-  auto split3 = [&](float rs) -> u32x4 {   // -rs as three binary16 terms in k-group 0
-    const _Float16 h0 = (_Float16)rs;
-    const float r1 = rs - (float)h0;
-    const _Float16 h1 = (_Float16)r1;
-    const _Float16 h2 = (_Float16)(r1 - (float)h1);
-    u32x4 r = {0u, 0u, 0u, 0u};
-    if (G == 0) {
-      r[0] = pack_h2(-(float)h0, -(float)h1);
-      r[1] = pack_h2(-(float)h2, 0.f);
-    }
-    return r;
-  };
-  const u32x4 corr_q = split3(rq), corr_do = split3(rd);
+  const bool big = offset_needs_x32(fmaxf(fabsf(rq), fabsf(rd)));
+  u32x4 corr_q = {0u, 0u, 0u, 0u}, corr_do = {0u, 0u, 0u, 0u};
+  if (G == 0) {
+    const u32x2 cq2 = offset_query_operand(rq, big), cd2 = offset_query_operand(rd, big);
+    corr_q[0] = cq2[0];
+    corr_q[1] = cq2[1];
+    corr_do[0] = cd2[0];
+    corr_do[1] = cd2[1];
+  }
   const float a_s = a.sm_scale_log2;
   const float nlse2 = q_ok ? -a.lse[tq0 + qi] * kLog2e : -INFINITY;   // padding rows: p = 0
 
@@ -173,11 +169,11 @@ template <typename S, int D> __global__ __launch_bounds__(256, 2) void skv_dq_ke
         f[rb] = mfma_h16(ca, qf[m], f[rb]);
         gq[rb] = mfma_h16(ca, dof[m], gq[rb]);
       }
-      const unsigned cz = magic_zp_pair(z_a[rb], z_a[rb]);
       u32x4 corr_k = {0u, 0u, 0u, 0u};
       if (G == 0) {
-        corr_k[0] = cz;
-        corr_k[1] = cz & 0xffffu;
+        const u32x2 ck2 = offset_key_operand(z_a[rb], big);
+        corr_k[0] = ck2[0];
+        corr_k[1] = ck2[1];
       }
       f[rb] = mfma_h16(corr_k, corr_q, f[rb]);
       gq[rb] = mfma_h16(corr_k, corr_do, gq[rb]);
@@ -411,7 +407,7 @@ template <typename S, int D, bool KEEP> __global__ __launch_bounds__(256, 2) voi
   // ---- this wave's tile in registers: code operands (B operands: column = key lr), scale, offset operand
   u32x4 cb[KD];
   float sk = 0.f;
-  u32x4 corr_k = {0u, 0u, 0u, 0u};
+  unsigned zw = 0u;   // this lane's zero point (low byte)
   auto expand_tile = [&]() {
     const int k_swz = KSW::swz(lr);
 #pragma unroll
@@ -421,14 +417,9 @@ template <typename S, int D, bool KEEP> __global__ __launch_bounds__(256, 2) voi
       cb[2 * jj + 1] = expand_codes(kw[2], kw[3]);
     }
     const unsigned *skp = reinterpret_cast<const unsigned *>(slot + SKV_TILE * D);
-    const unsigned skw = skp[lr], zw = skp[SKV_TILE + lr];
+    const unsigned skw = skp[lr];
+    zw = skp[SKV_TILE + lr];
     sk = std::is_same<S, float>::value ? __builtin_bit_cast(float, skw) : lo_to_f32<_Float16>(skw);
-    const unsigned cz = magic_zp_pair(zw, zw);
-    corr_k = u32x4{0u, 0u, 0u, 0u};
-    if (g == 0) {
-      corr_k[0] = cz;
-      corr_k[1] = cz & 0xffffu;
-    }
   };
 
   f32x16 dkv[DBW];
@@ -438,18 +429,20 @@ template <typename S, int D, bool KEEP> __global__ __launch_bounds__(256, 2) voi
     const float *stat = reinterpret_cast<const float *>(smem + SM::OFF_STAT) + (qb % NRB) * 128;
     const float a_sk = key_ok ? a.sm_scale_log2 * sk : 0.f;
     const float sm_k = key_ok ? a.sm_scale : 0.f;
-    auto split3 = [&](float rs) -> u32x4 {
-      const _Float16 h0 = (_Float16)rs;
-      const float r1 = rs - (float)h0;
-      const _Float16 h1 = (_Float16)r1;
-      const _Float16 h2 = (_Float16)(r1 - (float)h1);
-      u32x4 r = {0u, 0u, 0u, 0u};
-      if (g == 0) {
-        r[0] = pack_h2(-(float)h0, -(float)h1);
-        r[1] = pack_h2(-(float)h2, 0.f);
-      }
-      return r;
-    };
+    // operands of the rank-1 offset removal: one scaling for the whole query block
+    const float rs_q = stat[64 + lr], rs_do = stat[96 + lr];
+    const bool big = offset_needs_x32(fmaxf(fabsf(rs_q), fabsf(rs_do)));
+    u32x4 corr_q = {0u, 0u, 0u, 0u}, corr_do = {0u, 0u, 0u, 0u}, corr_k = {0u, 0u, 0u, 0u};
+    if (g == 0) {
+      const u32x2 cq2 = offset_query_operand(rs_q, big), cd2 = offset_query_operand(rs_do, big);
+      const u32x2 ck2 = offset_key_operand(zw, big);
+      corr_q[0] = cq2[0];
+      corr_q[1] = cq2[1];
+      corr_do[0] = cd2[0];
+      corr_do[1] = cd2[1];
+      corr_k[0] = ck2[0];
+      corr_k[1] = ck2[1];
+    }
     // S = Q C^T, dP = dO C^T (rows = queries, columns = keys), rank-1 offset removal
     f32x16 sacc, pacc;
 #pragma unroll
@@ -462,8 +455,8 @@ template <typename S, int D, bool KEEP> __global__ __launch_bounds__(256, 2) voi
       sacc = mfma_h(qa, cb[m], sacc);
       pacc = mfma_h(da, cb[m], pacc);
     }
-    sacc = mfma_h(split3(stat[64 + lr]), corr_k, sacc);
-    pacc = mfma_h(split3(stat[96 + lr]), corr_k, pacc);
+    sacc = mfma_h(corr_q, corr_k, sacc);
+    pacc = mfma_h(corr_do, corr_k, pacc);
     // p and ds for this lane's key; registers run over the queries 8aa + 4g + bb
     u32x4 pf[2], df[2];
 #pragma unroll

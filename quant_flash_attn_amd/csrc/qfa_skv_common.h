@@ -31,6 +31,30 @@ __device__ __forceinline__ unsigned pack_h2(float a, float b) { return pack2<_Fl
 __device__ __forceinline__ unsigned magic_zp_pair(unsigned za, unsigned zb) {
   return __builtin_amdgcn_perm(za, zb, 0x0c000c04u) ^ 0x64806480u;
 }
+// Operands of the rank-1 MFMA that removes the offset where codes are contracted over d:
+//     sum_d (1152 + c_jd) x_d  -  (1152 + zp_j) * rs,      rs = sum_d x_d.
+// The key side carries 1152 + zp_j in three k-slots, the query side -rs as three binary16 terms (33
+// significant bits, every product exact in fp32).  When some |rs| of the block reaches 2^15 (`big`, decided
+// for all queries of the MFMA together) the key side carries 32 * (1152 + zp_j) instead -- bits
+// 0x7800 | (zp_j + 128), still exact -- and the query side -rs / 32, which extends the range to 2^21.
+__device__ __forceinline__ bool offset_needs_x32(float rs) {
+  return __builtin_amdgcn_ballot_w64(!(fabsf(rs) < 32768.0f)) != 0;
+}
+// dwords 0 and 1 of the key-side operand (the caller zeroes them outside k-group 0; dwords 2, 3 are zero)
+__device__ __forceinline__ u32x2 offset_key_operand(unsigned z, bool big) {
+  const unsigned cz = __builtin_amdgcn_perm(z, z, 0x0c000c04u) ^ (big ? 0x78807880u : 0x64806480u);
+  return u32x2{cz, cz & 0xffffu};
+}
+// dwords 0 and 1 of the query-side operand
+__device__ __forceinline__ u32x2 offset_query_operand(float rs, bool big) {
+  const float x = big ? rs * 0.03125f : rs;
+  const _Float16 h0 = (_Float16)x;
+  const float r1 = x - (float)h0;
+  const _Float16 h1 = (_Float16)r1;
+  const _Float16 h2 = (_Float16)(r1 - (float)h1);
+  return u32x2{pack_h2(-(float)h0, -(float)h1), pack_h2(-(float)h2, 0.f)};
+}
+
 // ds_read_b64_tr_b8, issued like lds_read_tr16_async: invisible to the compiler's wait bookkeeping
 // (which would make it wait for every direct-to-LDS load in flight); use the result only after
 // lds_wait_all() and through tie().

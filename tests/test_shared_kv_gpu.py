@@ -344,3 +344,37 @@ def test_shared_kv_backward_strided_views(qfa, Nq):
     assert rc == 0, _lib.lib().qfa_last_error()
     torch.cuda.synchronize()
     assert torch.equal(dq_v, dq) and torch.equal(dkv_v, dkv)
+
+
+@pytest.mark.parametrize("Nq", [16, 40])
+def test_shared_kv_large_row_sums(qfa, Nq):
+    """Row sums of q beyond 2^15, where the rank-1 offset removal switches to its x32 scaling (without it the
+    correction operand overflows binary16 and O is NaN).  (c*q, sm_scale/c) is the same attention problem as
+    (q, sm_scale): O and dKV must not change and dQ must scale by 1/c, although the first run takes the x32
+    path and the second does not; both also match the fp64 oracle."""
+    B, H, Nk, D, c = 1, 2, 500, 128, 256.0
+    g = torch.Generator().manual_seed(17)
+    q = (2.0 + 0.1 * torch.randn((B, H, Nq, D), generator=g)).to(torch.float16)
+    kv = torch.randn((B, H, Nk, D), generator=g).to(torch.float16)
+    do = torch.randn((B, H, Nq, D), generator=g).to(torch.float16)
+    sm = 1.0 / math.sqrt(D)
+    qc = (q.float() * c).to(torch.float16)          # exact: a power of two
+    assert float(qc.float().sum(-1).abs().min()) > 32768.0 and float(q.float().sum(-1).abs().max()) < 32768.0
+    codes, scale, zp = qfa.asymmetric_quant_per_token(kv.to(DEV))
+    outs = []
+    for qq, s_ in ((q, sm), (qc, sm / c)):
+        o, lse = qfa.attn_fwd_shared_kv(qq.to(DEV), codes, scale, zp, s_)
+        dq, dkv = qfa.attn_bwd_shared_kv(qq.to(DEV), codes, scale, zp, o, do.to(DEV), lse, s_)
+        outs.append((o.cpu(), lse.cpu(), dq.cpu(), dkv.cpu()))
+    (o1, l1, dq1, dkv1), (o2, l2, dq2, dkv2) = outs
+    assert max_abs(o1, o2) <= 2.0 ** -9 * float(o1.abs().max()) and max_abs(l1, l2) < 1e-3
+    assert max_abs(dkv1, dkv2) <= 2e-3 * max(1.0, float(dkv1.abs().max()))
+    # dS is held in binary16 with sm_scale folded in: an sm_scale 256 times smaller than usual pushes it into
+    # the subnormal range, so dQ of the second run agrees to the gradient tolerance only
+    assert max_abs(dq1, dq2.float() * c) <= 2e-2 * max(1.0, float(dq1.abs().max()))
+    o_ref, lse_ref = oracle.legacy_fwd(qc, codes.cpu(), scale.cpu(), zp.cpu(), sm / c)
+    dq_ref, dkv_ref = oracle.legacy_bwd(qc, codes.cpu(), scale.cpu(), zp.cpu(), do, sm / c)
+    assert_close("O", o2, o_ref, scaled=True)
+    assert max_abs(l2, lse_ref) < LSE_TOL
+    assert_close("dQ", dq2.double() * c, dq_ref * c, scaled=True)
+    assert_close("dKV", dkv2, dkv_ref, scaled=True)
