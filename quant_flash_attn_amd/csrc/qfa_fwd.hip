@@ -25,9 +25,11 @@
 //
 // The kernel is bound by softmax VALU work, not by MFMA, so the design goal is to keep the vector
 // pipe busy and hide the matrix pipe under it:
-//  * the running maximum is only moved (and O rescaled) when some row of the wave exceeds it by
-//    more than 2^8 (any reference maximum gives the same O after the final division), so the
-//    rescale is a rare branch instead of 64 multiplies per tile;
+//  * the reference maximum is only moved (and O rescaled) when it has to be (any reference gives the
+//    same O after the final division): the masked loop moves it when a row exceeds it by more than
+//    2^8, the pipelined loop takes no maximum at all and watches the sum of each 16 probabilities
+//    instead (one compare; see check_half), so the rescale is a rare branch instead of 64 multiplies
+//    and 8 maxima per block;
 //  * row sums are taken over packed pairs with v_dot2;
 //  * tiles without any masked score run a software-pipelined loop whose body is one straight
 //    basic block per 32-key block: exp2/pack of block b, the P.V MFMAs of block b, the INT8 MFMAs
@@ -221,8 +223,8 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
   // move the reference maximum only when some row of the wave outgrew it by > 2^threshold
   // (the test is one compare against m_ref + threshold / a_i, kept in m_bound: it sits at the end
   // of a dependent chain that nothing else in the wave can overlap)
-  auto rescale_if_needed = [&](float mt) {
-    if (__builtin_amdgcn_ballot_w64(mt > m_bound) != 0) {
+  auto move_ref = [&](float mt) {
+    {
       const float m_new = fmaxf(m_ref, mt);
       const float alpha = __builtin_amdgcn_exp2f(a_i * (m_ref - m_new));
       m_ref = m_new;
@@ -234,6 +236,9 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) oacc[db][v] *= alpha;
     }
+  };
+  auto rescale_if_needed = [&](float mt) {
+    if (__builtin_amdgcn_ballot_w64(mt > m_bound) != 0) move_ref(mt);
   };
   // p = exp2(a_i*u - a_i*m_ref), packed; row sum; O^T += V^T . P^T for the 32 keys of block nb
   auto exp_pv = [&](int vbuf, int nb, const float (&u)[16]) {
@@ -316,20 +321,38 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
         vr[2 * db + 1] = lds_read_tr16_async<ROW0 + 8 * SM::VSTR>(ad);
       }
     };
-    auto exp_half = [&](int hh, u32x4 &pf) {
+    auto exp_half = [&](int hh, u32x4 &pf, float &lsum) {
+      lsum = 0.f;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, u[8 * hh + 2 * e], nm));
         const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, u[8 * hh + 2 * e + 1], nm));
         pf[e] = pack2<T>(p0, p1);
+        lsum = dot2_ones<T>(pf[e], lsum);   // sum of the rounded pair, fp32 accumulate
       }
+    };
+    // The pipelined loop takes no running maximum.  The probabilities of 16 keys are formed against the
+    // current reference and their sum is looked at before they reach the P.V MFMAs: only if some lane's
+    // sum left the range below (a score outgrew the reference by more than 2^60, or overflowed) is the
+    // maximum of the block taken, the reference moved (O and the row sum rescaled) and the 16
+    // probabilities formed again.  Any reference gives the same O after the final division.
+    constexpr float SUM_LIMIT = 0x1p60f;
+    auto check_half = [&](int hh, u32x4 &pf, float &lsum) {
+      if (__builtin_amdgcn_ballot_w64(!(lsum <= SUM_LIMIT)) != 0) {
+        float mt = -INFINITY;
+#pragma unroll
+        for (int v = 8 * hh; v < 16; ++v) mt = fmaxf(mt, u[v]);   // first half: the whole block
+        move_ref(max_across_halves(mt));
+        exp_half(hh, pf, lsum);
+      }
+      l_run += lsum;
     };
     // one body: V block (vbuf, nb); scores of the next block from kf; its constants in (cbuf, cnb);
     // then kf is refilled from K block (kbuf, knb).  `count_max`: whether the next block's maximum
     // may move the reference (false when that block belongs to a masked tile and is recomputed there).
     // `copy(i)`, i = 0..2, is called between phases: the steady loop issues one chunk of the next
     // tiles' copies there, so that the memory pipe sees single requests instead of a burst per tile
-    auto body = [&](int vbuf, auto nb_tag, int cbuf, int cnb, int kbuf, int knb, bool count_max, auto &&copy) {
+    auto body = [&](int vbuf, auto nb_tag, int cbuf, int cnb, int kbuf, int knb, auto &&copy) {
       static_assert(DB == 4 || DB == 2, "fragment arrays are sized for head_dim 128 or 64");
       u32x2 vr0[2 * DB], vr1[2 * DB];
       u32x4 pf0, pf1;
@@ -342,10 +365,12 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
       for (int v = 0; v < 16; ++v) s[v] = 0;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) s = mfma_i8(kf[ks], qf[ks], s);
-      if (!QK_ONLY) exp_half(0, pf0);
+      float l0, l1;
+      if (!QK_ONLY) exp_half(0, pf0, l0);
       __builtin_amdgcn_sched_barrier(0);
       copy(std::integral_constant<int, 0>{});
       if (!QK_ONLY) {
+        check_half(0, pf0, l0);
         v_frags(vbuf, NB, std::integral_constant<int, 1>{}, vr1);
         lds_wait_async<2 * DB>(vr0);   // the 2*DB requests just made may still be in flight
       }
@@ -361,10 +386,13 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
         for (int db = 0; db < DB; ++db)
           oacc[db] = mfma_16b<T>(u32x4{vr0[2 * db][0], vr0[2 * db][1], vr0[2 * db + 1][0], vr0[2 * db + 1][1]}, pf0,
                                  oacc[db]);
-        exp_half(1, pf1);
+        exp_half(1, pf1, l1);
       }
       __builtin_amdgcn_sched_barrier(0);
-      if (!QK_ONLY) lds_wait_async<0>(vr1);   // everything requested so far was requested a phase ago
+      if (!QK_ONLY) {
+        check_half(1, pf1, l1);
+        lds_wait_async<0>(vr1);   // everything requested so far was requested a phase ago
+      }
       copy(std::integral_constant<int, 1>{});
       k_frags(kbuf, knb);
       __builtin_amdgcn_sched_barrier(0);
@@ -385,24 +413,11 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
       __builtin_amdgcn_sched_barrier(0);
       copy(std::integral_constant<int, 2>{});
       f = mfma_16b<T>(corr_k, corr_q, f);
-      if (!QK_ONLY) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) l_run = dot2_ones<T>(pf0[e], l_run);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) l_run = dot2_ones<T>(pf1[e], l_run);
-      }
       __builtin_amdgcn_sched_barrier(0);
-      float mt0 = -INFINITY, mt1 = -INFINITY;   // two chains: half the dependent latency
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa)
 #pragma unroll
-        for (int bb = 0; bb < 4; ++bb) {
-          u[4 * aa + bb] = f[4 * aa + bb] * sk4[aa][bb];
-          if (aa & 1) mt1 = fmaxf(mt1, u[4 * aa + bb]);
-          else mt0 = fmaxf(mt0, u[4 * aa + bb]);
-        }
-      float mt = max_across_halves(fmaxf(mt0, mt1));
-      rescale_if_needed(count_max ? mt : -INFINITY);
+        for (int bb = 0; bb < 4; ++bb) u[4 * aa + bb] = f[4 * aa + bb] * sk4[aa][bb];
     };
 
     {   // block 0 prepared, fragments of block 1 in flight
@@ -429,9 +444,8 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
         if (i < KCH) cp_k.issue_one(rs_k, kd, wave_u, tid, i);
         else if (i < KCH + VCH) cp_v.issue_one(rs_v, vd, wave_u, tid, i - KCH);
       };
-      body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, true, [&](auto i) { chunk(decltype(i)::value); });
-      body(t & 1, std::integral_constant<int, 1>{}, kb_nxt, 0, kb_nxt, 1, t + 1 < t_hot,
-           [&](auto i) { chunk(3 + decltype(i)::value); });
+      body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, [&](auto i) { chunk(decltype(i)::value); });
+      body(t & 1, std::integral_constant<int, 1>{}, kb_nxt, 0, kb_nxt, 1, [&](auto i) { chunk(3 + decltype(i)::value); });
       static_assert(KCH + VCH <= 6, "six copy slots per tile");
       store_k(kb_free);
       const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
@@ -441,8 +455,8 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
     for (; t < t_hot; ++t) {
       if (t + 2 < ntiles) load_k(t + 2, kb_free);
       if (t + 1 < ntiles) load_v(t + 1);
-      body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, true, no_copy);
-      body(t & 1, std::integral_constant<int, 1>{}, kb_nxt, 0, kb_nxt, 1, t + 1 < t_hot, no_copy);
+      body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, no_copy);
+      body(t & 1, std::integral_constant<int, 1>{}, kb_nxt, 0, kb_nxt, 1, no_copy);
       if (t + 2 < ntiles) store_k(kb_free);
       const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
       dma_wait();

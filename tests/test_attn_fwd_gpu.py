@@ -61,6 +61,32 @@ def test_forward_vs_oracle(qfa, B, H, Nq, Nk, D, causal, config, dtype):
     assert torch.equal(qq.codes.cpu(), oracle.quantize_per_token_c(q)[0])
 
 
+@pytest.mark.parametrize("D,dtype", [(128, torch.bfloat16), (64, torch.float16)])
+@pytest.mark.parametrize("jump", [64, 80, 104, 352])
+@pytest.mark.parametrize("causal", [False, True])
+def test_scores_jump_far_above_the_running_reference(qfa, D, dtype, jump, causal):
+    """Keys from index `jump` on score hundreds of nats above the earlier ones.  The pipelined loop keeps no
+    running maximum; it must notice (from the sum of 16 probabilities, before they are multiplied with V) that
+    its reference is stale and move it -- in the first or the second half of a 32-key block, depending on
+    where the jump sits -- and the earlier keys' contribution must vanish cleanly instead of turning into
+    inf/NaN."""
+    B, H, N = 1, 2, 512
+    g = torch.Generator().manual_seed(jump + D)
+    q = (3.0 + 0.3 * torch.randn((B, H, N, D), generator=g)).to(dtype)
+    k = 0.1 * torch.randn((B, H, N, D), generator=g)
+    k[:, :, jump:] += 3.0
+    k[:, 1, jump + 200:] += 2.0          # a second jump in one head
+    k = k.to(dtype)
+    v = torch.randn((B, H, N, D), generator=g).to(dtype)
+    sm = 1.0 / math.sqrt(D)
+    qq, kq, o, lse = _run(qfa, q, k, v, causal, sm)
+    o_ref, lse_ref = _oracle_fwd(qq, kq, v, causal, sm)
+    sc = sm * (q[0, 0].double() @ k[0, 0].double().T)
+    assert float(sc[:, jump:].min() - sc[:, :jump].max()) > 60.0 * math.log(2.0)   # more than 2^60 apart
+    assert_close("O", o.cpu(), o_ref)
+    assert max_abs(lse.cpu(), lse_ref) < LSE_TOL * max(1.0, float(lse_ref.abs().max()) / 64)
+
+
 def test_fp32_plumbing_configuration(qfa):
     """B1 H4 N256 D64 fp32 q,k,v, seed 0, non-causal, through the autograd entry point."""
     torch.manual_seed(0)
