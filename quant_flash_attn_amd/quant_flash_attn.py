@@ -10,7 +10,7 @@ Two autograd entry points, both backed by the HIP kernels behind qfa_attn_fwd / 
   QuantFlashAttention.apply(q, kv_fp16, kv_quant, sm_scale)     (alias quant_flash_attn)
       The reference's own entry point (quant_flash_attn.py:173-240): one quantized tensor serves as
       K and V, `kv_fp16` only receives the gradient, backward returns (dq, dkv, None, None) with
-      dkv = dK + dV (:161).  Query blocks of up to SHARED_KV_MAX_Q (512) tokens run the reference's
+      dkv = dK + dV (:161).  Query blocks of up to SHARED_KV_MAX_Q (512) tokens (any length at head_dim 256) run the reference's
       computation itself in the forward (Q in 16-bit, qfa_attn_fwd_shared_kv) and in the backward
       (qfa_attn_bwd_shared_kv, binary16 arithmetic; bf16 tensors are converted around it).  Longer
       query blocks go through the INT8-score kernels, where Q is quantized per token too (stated
@@ -263,7 +263,8 @@ class QuantFlashAttention(torch.autograd.Function):
             raise ValueError(f"shape mismatch: q {tuple(q.shape)}, kv {tuple(kv_fp16.shape)}, codes {tuple(codes.shape)}")
         ctx.sm_scale = float(sm_scale)
         ctx.q_dtype, ctx.kv_dtype = q.dtype, kv_fp16.dtype
-        ctx.shared_kv = q.shape[2] <= SHARED_KV_MAX_Q and q.dtype in _IO_DTYPES
+        # head_dim 256 (compute_flops.py:94) exists only in the shared-KV kernels: any Nq goes there
+        ctx.shared_kv = (q.shape[2] <= SHARED_KV_MAX_Q or q.shape[3] == 256) and q.dtype in _IO_DTYPES
         if ctx.shared_kv:
             # the reference's computation itself: Q unquantized, the codes streamed once (:50-69)
             o, lse = attn_fwd_shared_kv(q, codes, scale, zp, sm_scale)

@@ -161,6 +161,26 @@ def test_shared_kv_entry_point_long_query_block(qfa):
     assert_close("dKV", kvd.grad.cpu(), dkv_ref, scaled=True)
 
 
+def test_entry_point_head_dim_256_beyond_the_query_limit(qfa):
+    """600 queries at head_dim 256: longer than the query blocks the shared-KV kernels are normally given, but
+    the INT8-score kernels stop at head_dim 128, so the reference's entry point keeps them on this path."""
+    B, H, Nq, Nk, D = 1, 2, 600, 700, 256
+    q, kv = _inputs("normal", B, H, Nq, Nk, D, torch.float16, seed=21)
+    sm = 1.0 / math.sqrt(D)
+    qd = q.to(DEV).requires_grad_(True)
+    kvd = kv.to(DEV).requires_grad_(True)
+    kv_quant = qfa.asymmetric_quant_per_token(kvd.detach())
+    o = qfa.quant_flash_attn(qd, kvd, kv_quant, sm)
+    do = torch.randn(o.shape, generator=torch.Generator().manual_seed(4)).to(torch.float16)
+    o.backward(do.to(DEV))
+    codes, scale, zp = (t.cpu() for t in kv_quant)
+    o_ref, _ = oracle.legacy_fwd(q, codes, scale, zp, sm)
+    dq_ref, dkv_ref = oracle.legacy_bwd(q, codes, scale, zp, do, sm)
+    assert_close("O", o.detach().cpu(), o_ref, scaled=True)
+    assert_close("dQ", qd.grad.cpu(), dq_ref, scaled=True)
+    assert_close("dKV", kvd.grad.cpu(), dkv_ref, scaled=True)
+
+
 @pytest.mark.parametrize("B,H,Nq,Nk,D", [(1, 2, 16, 4096, 128), (1, 1, 1, 20000, 64), (2, 3, 40, 3001, 128), (1, 8, 5, 1023, 64)])
 def test_shared_kv_forward_split_over_keys(qfa, B, H, Nq, Nk, D):
     """Few (batch, head) pairs: the wrapper hands the library a workspace and the keys of a query block are
