@@ -444,8 +444,9 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(BwdArgs a) {
 //   dS-wave (w >= 4): dP = dO.V^T, then dS' = P o (dP - delta) * a with the partner's P,
 //                     dK^T += Qz^T.dS'
 // No product is computed twice, each wave keeps 64 accumulator registers, and within a SIMD one wave
-// is in its VALU phase while the other feeds the matrix pipe.  Two barriers per 32-query block: after
-// P is written, and after it has been consumed.
+// is in its VALU phase while the other feeds the matrix pipe.  One barrier per 32-query block: P goes
+// to the exchange slot of the block's parity, so the slot written for block b is read before barrier
+// b+1 and not written again before that barrier has passed.
 constexpr int DKV_THREADS = 512;
 
 template <typename T, int D, bool CAUSAL>
