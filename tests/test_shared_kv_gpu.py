@@ -161,6 +161,36 @@ def test_shared_kv_entry_point_long_query_block(qfa):
     assert_close("dKV", kvd.grad.cpu(), dkv_ref, scaled=True)
 
 
+@pytest.mark.parametrize("B,H,Nq,Nk,D,seed", [(1, 1, 5, 32, 128, 1158), (1, 3, 5, 33, 256, 1114), (1, 1, 130, 32, 256, 1091),
+                                             (2, 2, 17, 1025, 256, 1068)])
+def test_nearly_one_hot_softmax_gradient_floor(qfa, B, H, Nq, Nk, D, seed):
+    """Scores that grow along the keys make the softmax nearly one-hot; dQ = sm * dS K is then a small
+    difference of large terms and the 16-bit rounding of O (which enters delta = rowsum(O o dO), in the
+    reference too: quant_flash_attn.py:97-99) alone moves it by a fifth of its size, so the cosine against
+    an exact backward says nothing.  The bar here: the error stays within a small multiple of what that
+    rounding causes in an otherwise exact fp64 backward, and within the absolute gradient tolerance."""
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn((B, H, Nq, D), generator=g) * 0.2 + 1.0
+    kv = torch.randn((B, H, Nk, D), generator=g) * 0.3 + torch.linspace(-1, 3, Nk).view(1, 1, Nk, 1)
+    do = torch.randn((B, H, Nq, D), generator=g)
+    q, kv, do = q.half(), kv.half(), do.half()
+    sm = 1.0 / math.sqrt(D)
+    codes, scale, zp = qfa.asymmetric_quant_per_token(kv.to(DEV))
+    o, lse = qfa.attn_fwd_shared_kv(q.to(DEV), codes, scale, zp, sm)
+    dq, dkv = qfa.attn_bwd_shared_kv(q.to(DEV), codes, scale, zp, o, do.to(DEV), lse, sm)
+    c, s_, z = codes.cpu(), scale.cpu(), zp.cpu()
+    dq_ref, dkv_ref = oracle.legacy_bwd(q, c, s_, z, do, sm)
+    kvh = (c.double() - z.double()) * s_.double()
+    P = torch.softmax(sm * (q.double() @ kvh.transpose(-1, -2)), -1)
+    delta16 = ((P @ kvh).half().double() * do.double()).sum(-1, keepdim=True)     # the only rounding kept
+    dq_floor = sm * (P * (do.double() @ kvh.transpose(-1, -2) - delta16)) @ kvh
+    floor = max_abs(dq_floor, dq_ref)
+    err = max_abs(dq.cpu(), dq_ref)
+    assert err <= 3.0 * floor + 2.0 ** -11 * float(dq_ref.abs().max()) + 1e-4, (err, floor)
+    assert err <= 2e-2 * max(1.0, float(dq_ref.abs().max()))
+    assert_close("dKV", dkv.cpu(), dkv_ref, scaled=True)
+
+
 def test_entry_point_head_dim_256_beyond_the_query_limit(qfa):
     """600 queries at head_dim 256: longer than the query blocks the shared-KV kernels are normally given, but
     the INT8-score kernels stop at head_dim 128, so the reference's entry point keeps them on this path."""
