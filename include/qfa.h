@@ -138,7 +138,7 @@ int qfa_attn_fwd_shared_kv(const void *q, const int8_t *codes, const void *scale
  *   grad_scale  nullable DEVICE pointer to one float that multiplies dq and dkv before they are rounded.
  *               dQ and dKV are linear in dO: a caller whose dO does not fit binary16 (bf16 training) hands
  *               over dO * 2^k and *grad_scale = 2^-k without a host synchronisation;
- *   codes, scale, scale_dtype, zp, lse as in the forward.  D in {64, 128, 256} (256: always the two kernels).
+ *   codes, scale, scale_dtype, zp, lse as in the forward.  D in {64, 128, 256} (256: one pass up to 16 queries).
  *   The sums of a query's and of a dO row's D elements must stay inside binary16 range.
  */
 int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp,

@@ -198,7 +198,9 @@ int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale
   if (sqn >= (1 << 23) || son >= (1 << 23) || sdon >= (1 << 23))
     return set_error(QFA_EUNSUPPORTED, "%s: token strides of 2^23 elements or more are not supported", who);
   // one fused pass keeps a (batch, head)'s dQ in registers: at most 32 queries, head_dim up to 128
-  return Nq <= 32 && D <= 128 ? launch_skv_bwd(a, (hipStream_t)stream) : launch_skv_bwd_long(a, (hipStream_t)stream);
+  // one fused pass while the per-wave accumulators fit: 32 queries up to head_dim 128, 16 at 256
+  const bool one_pass = (Nq <= 32 && D <= 128) || (Nq <= 16 && D == 256);
+  return one_pass ? launch_skv_bwd(a, (hipStream_t)stream) : launch_skv_bwd_long(a, (hipStream_t)stream);
 }
 
 int qfa_bench_qk_stage(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,

@@ -72,7 +72,7 @@ template <int OFF> __device__ __forceinline__ u32x2 lds_tr16(unsigned addr) { re
 
 // S: element type of the scale vector (float or _Float16).  HALF: at most 16 queries -- rows 16..31 of the
 // query block are padding, so their share of steps 2 and 4 is skipped (P and dS are zero there).
-template <typename S, int D, bool HALF> __global__ __launch_bounds__(256, 2) void skv_bwd_kernel(SkvBwdArgs a) {
+template <typename S, int D, bool HALF> __global__ __launch_bounds__(256, D == 256 ? 1 : 2) void skv_bwd_kernel(SkvBwdArgs a) {
   constexpr int QH = HALF ? 1 : 2;   // 16-query halves of the block that hold queries
   typedef SkvBwdSmem<D> SM;
   typedef Swz<D> KSW;
@@ -430,7 +430,8 @@ template <typename S, int D> static int launch_skv_bwd_sd(const SkvAttnArgs &x, 
   const int64_t total = x.B * x.H;
   if (total > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "attn_bwd_shared_kv: too many (batch, head) pairs for one launch");
   if (x.Nq <= 16) skv_bwd_kernel<S, D, true><<<dim3((unsigned)total), dim3(256), 0, st>>>(a);
-  else skv_bwd_kernel<S, D, false><<<dim3((unsigned)total), dim3(256), 0, st>>>(a);
+  else if constexpr (D <= 128) skv_bwd_kernel<S, D, false><<<dim3((unsigned)total), dim3(256), 0, st>>>(a);
+  else return set_error(QFA_EUNSUPPORTED, "attn_bwd_shared_kv: the one-pass kernel takes at most 16 queries at head_dim 256");
   return check_launch("qfa_attn_bwd_shared_kv");
 }
 
@@ -438,7 +439,8 @@ int launch_skv_bwd(const SkvAttnArgs &x, hipStream_t st) {
   const bool s32 = x.scale_dtype == QFA_F32;
   if (x.D == 128) return s32 ? launch_skv_bwd_sd<float, 128>(x, st) : launch_skv_bwd_sd<_Float16, 128>(x, st);
   if (x.D == 64) return s32 ? launch_skv_bwd_sd<float, 64>(x, st) : launch_skv_bwd_sd<_Float16, 64>(x, st);
-  return set_error(QFA_EUNSUPPORTED, "attn_bwd_shared_kv: head_dim must be 64 or 128");
+  if (x.D == 256) return s32 ? launch_skv_bwd_sd<float, 256>(x, st) : launch_skv_bwd_sd<_Float16, 256>(x, st);
+  return set_error(QFA_EUNSUPPORTED, "attn_bwd_shared_kv: head_dim must be 64, 128 or 256");
 }
 
 }  // namespace qfa

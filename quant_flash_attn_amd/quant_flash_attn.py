@@ -171,7 +171,7 @@ def attn_bwd_shared_kv(q: torch.Tensor, codes: torch.Tensor, scale: torch.Tensor
     (quant_flash_attn.py:104-166) with dKV = dV + dK as stored there (:161).  q, o, do fp16
     [B,H,Nq,D] (the kernels compute in binary16); lse as returned by the forward.  dQ and dKV come back
     in `grad_dtype` (fp16 by default, or bf16), multiplied by the one-element device tensor `grad_scale`
-    if given.  Up to 32 queries run in one fused pass over the codes, longer blocks (and head_dim 256)
+    if given.  Up to 32 queries (16 at head_dim 256) run in one fused pass over the codes, longer blocks
     in a dQ kernel plus a dKV kernel."""
     if q.dtype != torch.float16 or o.dtype != torch.float16:
         raise TypeError("the shared-KV backward kernel computes in float16: q and o must be float16")

@@ -70,7 +70,8 @@ BWD_CASES = [
     (1, 3, 33, 100, 64, "offset", torch.float32),        # one query past a block, one key chunk
     (1, 2, 128, 1000, 128, "uniform", torch.float16),
     (2, 2, 64, 129, 64, "outlier", torch.float32),       # second key chunk holds a single key
-    # head_dim 256 (compute_flops.py:94): always the two kernels, two waves share a tile in the dKV kernel
+    # head_dim 256 (compute_flops.py:94): one pass up to 16 queries; beyond, the two kernels (two waves share
+    # a tile in the dKV kernel)
     (2, 2, 16, 3000, 256, "normal", torch.float16),
     (1, 2, 70, 161, 256, "offset", torch.float32),
     (1, 1, 1, 1, 256, "normal", torch.float16),
