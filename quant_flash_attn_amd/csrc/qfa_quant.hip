@@ -132,11 +132,11 @@ template <typename T, int D, int U> __global__ __launch_bounds__(256) void quant
       q = __builtin_fmaf(__builtin_fmaf(-scale, q, x), r, q);
       return q;
     };
-    // roundf (ties away from zero): trunc, exact fraction, compare with one half
+    // roundf (ties away from zero) in three instructions: add the largest float below one half with the
+    // sign of y, truncate.  Equal to roundf for every binary32 value (checked exhaustively on the CPU; the
+    // classic y + 0.5 fails at 0.49999997).
     auto round_away = [](float y) -> float {
-      const float t = __builtin_truncf(y);
-      const float d = y - t;
-      return (fabsf(d) >= 0.5f) ? t + __builtin_copysignf(1.0f, y) : t;
+      return __builtin_truncf(y + __builtin_copysignf(0x1.fffffep-2f, y));
     };
     float q[8], qmn;
     if (fast) {
