@@ -19,27 +19,40 @@
 
 namespace qfa {
 
+// One reduction step = one instruction: the lane permute is the DPP modifier of the min / max itself.
+// (Written as asm: through the builtin the permuted value comes back as an integer, and the compiler
+// then spends a v_mov_b32_dpp and a canonicalising v_max on every step.  The s_nop covers the two wait
+// states a DPP read needs after a vector write of the same register, which the compiler does not
+// insert for instructions it cannot see.)
+#define QFA_DPP_STEP(OP, CTRL)                                                                           \
+  asm("s_nop 1\n\t" OP " %0, %1, %1 " CTRL " row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v))
 template <int LPT> __device__ __forceinline__ float group_min(float v) {
-  v = fminf(v, dpp_f<0xB1>(v));
-  if (LPT >= 4) v = fminf(v, dpp_f<0x4E>(v));
-  if (LPT >= 8) v = fminf(v, dpp_f<0x141>(v));
-  if (LPT >= 16) v = fminf(v, dpp_f<0x140>(v));
+  float r;
+  QFA_DPP_STEP("v_min_f32_dpp", "quad_perm:[1,0,3,2]"); v = r;
+  if (LPT >= 4) { QFA_DPP_STEP("v_min_f32_dpp", "quad_perm:[2,3,0,1]"); v = r; }
+  if (LPT >= 8) { QFA_DPP_STEP("v_min_f32_dpp", "row_half_mirror"); v = r; }
+  if (LPT >= 16) { QFA_DPP_STEP("v_min_f32_dpp", "row_mirror"); v = r; }
   if (LPT >= 32) v = fminf(v, __shfl_xor(v, 16, 64));
   return v;
 }
 template <int LPT> __device__ __forceinline__ float group_max(float v) {
-  v = fmaxf(v, dpp_f<0xB1>(v));
-  if (LPT >= 4) v = fmaxf(v, dpp_f<0x4E>(v));
-  if (LPT >= 8) v = fmaxf(v, dpp_f<0x141>(v));
-  if (LPT >= 16) v = fmaxf(v, dpp_f<0x140>(v));
+  float r;
+  QFA_DPP_STEP("v_max_f32_dpp", "quad_perm:[1,0,3,2]"); v = r;
+  if (LPT >= 4) { QFA_DPP_STEP("v_max_f32_dpp", "quad_perm:[2,3,0,1]"); v = r; }
+  if (LPT >= 8) { QFA_DPP_STEP("v_max_f32_dpp", "row_half_mirror"); v = r; }
+  if (LPT >= 16) { QFA_DPP_STEP("v_max_f32_dpp", "row_mirror"); v = r; }
   if (LPT >= 32) v = fmaxf(v, __shfl_xor(v, 16, 64));
   return v;
 }
+#undef QFA_DPP_STEP
+// integer sum: `old` = 0, the identity of the addition (never used: every lane reads a valid lane),
+// lets the compiler fold the permute into v_add_u32_dpp
+template <int CTRL> __device__ __forceinline__ int dpp_zero(int x) { return __builtin_amdgcn_update_dpp(0, x, CTRL, 0xf, 0xf, false); }
 template <int LPT> __device__ __forceinline__ int group_sum(int v) {
-  v += dpp_i<0xB1>(v);
-  if (LPT >= 4) v += dpp_i<0x4E>(v);
-  if (LPT >= 8) v += dpp_i<0x141>(v);
-  if (LPT >= 16) v += dpp_i<0x140>(v);
+  v += dpp_zero<0xB1>(v);
+  if (LPT >= 4) v += dpp_zero<0x4E>(v);
+  if (LPT >= 8) v += dpp_zero<0x141>(v);
+  if (LPT >= 16) v += dpp_zero<0x140>(v);
   if (LPT >= 32) v += __shfl_xor(v, 16, 64);
   return v;
 }
