@@ -97,10 +97,11 @@ def test_shared_kv_backward_vs_oracle(qfa, B, H, Nq, Nk, D, config, sdtype):
     assert_close("dKV", dkv.cpu(), dkv_ref, scaled=True)
 
 
-def test_shared_kv_entry_point_autograd(qfa):
-    """The reference's entry point end to end on its benchmark shape (small batch): forward and
-    backward run the shared-KV kernels and kv_fp16 receives dKV (quant_flash_attn.py:178-237)."""
-    B, H, Nq, Nk, D = 2, 4, 16, 3000, 128
+@pytest.mark.parametrize("D", [128, 256, 64])
+def test_shared_kv_entry_point_autograd(qfa, D):
+    """The reference's entry point end to end on its benchmark shapes (compute_flops.py:94-96, small batch):
+    forward and backward run the shared-KV kernels and kv_fp16 receives dKV (quant_flash_attn.py:178-237)."""
+    B, H, Nq, Nk = 2, 4, 16, 3000
     q, kv = _inputs("normal", B, H, Nq, Nk, D, torch.float16, seed=11)
     sm = 1.0 / math.sqrt(D)
     qd = q.to(DEV).requires_grad_(True)
@@ -118,12 +119,12 @@ def test_shared_kv_entry_point_autograd(qfa):
     assert kvd.grad.dtype == torch.float16 and qd.grad.dtype == torch.float16
 
 
-@pytest.mark.parametrize("do_scale", [1.0, 2.0 ** -22])
-def test_shared_kv_entry_point_bf16(qfa, do_scale):
+@pytest.mark.parametrize("do_scale,D", [(1.0, 128), (2.0 ** -22, 128), (1.0, 256)])
+def test_shared_kv_entry_point_bf16(qfa, do_scale, D):
     """bf16 tensors through the reference's entry point: forward in the shared-KV kernel (queries rounded to
     binary16), backward in the binary16 kernels with dO scaled into range by a power of two -- also when
     dO is far below binary16's smallest normal number."""
-    B, H, Nq, Nk, D = 2, 3, 16, 700, 128
+    B, H, Nq, Nk = 2, 3, 16, 700
     q, kv = _inputs("normal", B, H, Nq, Nk, D, torch.bfloat16, seed=31)
     sm = 1.0 / math.sqrt(D)
     qd = q.to(DEV).requires_grad_(True)
