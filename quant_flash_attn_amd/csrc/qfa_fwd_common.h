@@ -16,6 +16,7 @@ struct FwdArgs {
   int mblocks;           // query blocks of one workgroup each per (batch, head)
   int total_blocks;      // mblocks * B * H
   int blocks_per_xcd;    // ceil(total_blocks / 8)
+  int group_log2;        // causal: log2 of the number of heads whose query blocks are dispatched together
 };
 
 #ifndef QFA_FWD_WAVES
