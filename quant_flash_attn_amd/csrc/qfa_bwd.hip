@@ -269,9 +269,19 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(BwdArgs a) {
   const int L = blockIdx.x;
   const int vid = (L % 8) * a.blocks_per_xcd + (L / 8);
   if (vid >= a.total_blocks) return;
-  const int bh = vid / a.nblocks;
+  int bh = vid / a.nblocks;
   int mb = vid % a.nblocks;
-  if (CAUSAL) mb = a.nblocks - 1 - mb;
+  if (CAUSAL) {
+    // longest rows first, two heads at a time (ids alternate between the heads of a pair): with one head
+    // after the other the last head's long blocks start while the chip is already draining
+    const int pb = bh & ~1;
+    if (pb + 2 <= a.total_blocks / a.nblocks) {
+      const int idx = (bh - pb) * a.nblocks + mb;
+      bh = pb + (idx & 1);
+      mb = idx >> 1;
+    }
+    mb = a.nblocks - 1 - mb;
+  }
   const int64_t b = bh / a.H, h = bh % a.H;
   const int m0 = mb * DQ_BLK;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, lr = lane % 32, g = lane / 32;
