@@ -114,6 +114,7 @@ struct BwdArgs {
   float sm_scale, sm_scale_log2;
   int nblocks;          // query blocks (dq) or key blocks (dkdv) per (b,h)
   int total_blocks, blocks_per_xcd;
+  int group_log2;       // dkdv, causal: log2 of the number of heads whose key blocks are dispatched together
 };
 
 // position of streamed row r (0..63) inside a transposed tile: the order in which the 32x32
@@ -475,8 +476,19 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
   const int L = blockIdx.x;
   const int vid = (L % 8) * a.blocks_per_xcd + (L / 8);
   if (vid >= a.total_blocks) return;
-  const int bh = vid / a.nblocks;
-  const int nbk = vid % a.nblocks;   // causal: early key blocks see the most queries and come first
+  int bh = vid / a.nblocks;
+  int nbk = vid % a.nblocks;   // causal: early key blocks see the most queries and come first
+  if (CAUSAL && a.group_log2 > 0) {
+    // key blocks of 2^group_log2 heads dispatched together, from the longest down (as in the dQ kernel);
+    // the launcher allows it only while the query-side tiles of the group fit an XCD's L2
+    const int GL = a.group_log2;
+    const int pb = bh >> GL << GL;
+    if (pb + (1 << GL) <= a.total_blocks / a.nblocks) {
+      const int idx = (bh - pb) * a.nblocks + nbk;
+      bh = pb + (idx & ((1 << GL) - 1));
+      nbk = idx >> GL;
+    }
+  }
   const int64_t b = bh / a.H, h = bh % a.H;
   const int n0 = nbk * BWD_BLK;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, lr = lane % 32, g = lane / 32;
@@ -760,7 +772,7 @@ template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStre
   a.sdob = x.sdob; a.sdoh = x.sdoh; a.sdon = x.sdon; a.sdqb = x.sdqb; a.sdqh = x.sdqh; a.sdqn = x.sdqn;
   a.sdkb = x.sdkb; a.sdkh = x.sdkh; a.sdkn = x.sdkn; a.sdvb = x.sdvb; a.sdvh = x.sdvh; a.sdvn = x.sdvn;
   a.sm_scale = x.sm_scale; a.sm_scale_log2 = x.sm_scale * kLog2e;
-  a.nblocks = 0; a.total_blocks = 0; a.blocks_per_xcd = 0;
+  a.nblocks = 0; a.total_blocks = 0; a.blocks_per_xcd = 0; a.group_log2 = 0;
   const dim3 block(256);
   const int64_t BH = x.B * x.H;
   if (BH * a.tiles_q > 0x7fffffffLL || BH * a.tiles_k > 0x7fffffffLL)
@@ -773,6 +785,11 @@ template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStre
   // dK, dV
   {
     a.nblocks = (int)((x.Nk + BWD_BLK - 1) / BWD_BLK);
+    // per head the kernel streams Qc, dO, dO^T and Qz^T (7 bytes per query and d): group heads while that
+    // stays within an XCD's 4 MB L2 (one head already fills it at N=4096, D=128)
+    const int64_t head_bytes = x.Nq * (int64_t)D * 7;
+    a.group_log2 = 0;
+    while (a.group_log2 < 2 && (head_bytes << (a.group_log2 + 1)) <= (4 << 20)) ++a.group_log2;
     const int64_t total = (int64_t)a.nblocks * BH;
     if (total > 0x3fffffffLL) return set_error(QFA_EUNSUPPORTED, "attn_bwd: too many key blocks for one launch");
     a.total_blocks = (int)total;
