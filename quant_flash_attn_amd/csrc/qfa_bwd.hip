@@ -114,7 +114,7 @@ struct BwdArgs {
   float sm_scale, sm_scale_log2;
   int nblocks;          // query blocks (dq) or key blocks (dkdv) per (b,h)
   int total_blocks, blocks_per_xcd;
-  int group_log2;       // dkdv, causal: log2 of the number of heads whose key blocks are dispatched together
+  int group_log2;       // causal: log2 of the number of heads whose blocks are dispatched together (set per launch)
 };
 
 // position of streamed row r (0..63) inside a transposed tile: the order in which the 32x32
@@ -273,13 +273,14 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(BwdArgs a) {
   int bh = vid / a.nblocks;
   int mb = vid % a.nblocks;
   if (CAUSAL) {
-    // longest rows first, two heads at a time (ids alternate between the heads of a pair): with one head
-    // after the other the last head's long blocks start while the chip is already draining
-    const int pb = bh & ~1;
-    if (pb + 2 <= a.total_blocks / a.nblocks) {
+    // longest rows first, 2^group_log2 heads at a time (ids cycle through the heads of a group): with one
+    // head after the other the last head's long blocks start while the chip is already draining
+    const int GL = a.group_log2;
+    const int pb = bh >> GL << GL;
+    if (pb + (1 << GL) <= a.total_blocks / a.nblocks) {
       const int idx = (bh - pb) * a.nblocks + mb;
-      bh = pb + (idx & 1);
-      mb = idx >> 1;
+      bh = pb + (idx & ((1 << GL) - 1));
+      mb = idx >> GL;
     }
     mb = a.nblocks - 1 - mb;
   }
@@ -802,6 +803,11 @@ template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStre
   // dQ
   {
     a.nblocks = (int)((x.Nq + DQ_BLK - 1) / DQ_BLK);
+    // per head the kernel streams Kc, V and Kz^T (5 bytes per key and d): two to eight heads together, within
+    // about 6 MB (pairs at N=4096, D=128, measured)
+    const int64_t head_bytes_k = x.Nk * (int64_t)D * 5;
+    a.group_log2 = 1;
+    while (a.group_log2 < 3 && (head_bytes_k << (a.group_log2 + 1)) <= (6 << 20)) ++a.group_log2;
     const int64_t total = (int64_t)a.nblocks * BH;
     if (total > 0x3fffffffLL) return set_error(QFA_EUNSUPPORTED, "attn_bwd: too many query blocks for one launch");
     a.total_blocks = (int)total;
