@@ -42,6 +42,11 @@ CASES = [
     (1, 3, 333, 333, 64, True, "uniform", torch.bfloat16),      # ragged, causal
     (2, 2, 97, 689, 128, False, "normal", torch.bfloat16),      # short Q, long ragged KV
     (1, 2, 640, 640, 128, True, "offset", torch.float16),
+    # causal with many heads: the kernels dispatch the blocks of a group of heads together; 12 and 19 heads
+    # leave a partial group at the end, 16 fills two groups of eight
+    (3, 4, 320, 320, 64, True, "normal", torch.bfloat16),
+    (1, 19, 300, 300, 128, True, "offset", torch.bfloat16),
+    (2, 8, 512, 512, 64, True, "uniform", torch.float16),
 ]
 
 

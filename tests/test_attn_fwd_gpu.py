@@ -43,6 +43,10 @@ CASES = [
     (2, 2, 97, 689, 128, False, "normal", torch.bfloat16),      # short Q, long ragged KV (reference test shape)
     (1, 2, 17, 1023, 128, False, "normal", torch.float16),
     (1, 2, 640, 640, 128, True, "offset", torch.float16),
+    # causal with many heads: query blocks of a group of heads are dispatched together; 12 and 19 heads leave
+    # a partial group at the end
+    (3, 4, 320, 320, 64, True, "normal", torch.bfloat16),
+    (1, 19, 300, 300, 128, True, "offset", torch.bfloat16),
 ]
 
 
