@@ -313,7 +313,9 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
     //   exp2/pack and P.V of block b | INT8 product of block b+1 | convert/correct/scale/max of b+1,
     // with every LDS operand requested a phase (or a body) before the MFMA that consumes it.  The
     // phases are fenced so that the requests stay where they are; inside a phase MFMA and VALU
-    // instructions are independent and interleave.
+    // instructions are independent and interleave.  A wave raises its issue priority for the phases that
+    // hold MFMAs and drops it for the ones that wait and request, so that of the two waves of a SIMD the
+    // one that can feed the matrix pipe goes first (2 % at the non-causal sizes, nothing at the causal ones).
     // Carried between bodies: u = prepared scores of block b, kf = K fragments of block b+1.
     float u[16];
     i32x4 kf[KS];
@@ -362,8 +364,7 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
       l_run += lsum;
     };
     // one body: V block (vbuf, nb); scores of the next block from kf; its constants in (cbuf, cnb);
-    // then kf is refilled from K block (kbuf, knb).  `count_max`: whether the next block's maximum
-    // may move the reference (false when that block belongs to a masked tile and is recomputed there).
+    // then kf is refilled from K block (kbuf, knb).
     // `copy(i)`, i = 0..2, is called between phases: the steady loop issues one chunk of the next
     // tiles' copies there, so that the memory pipe sees single requests instead of a burst per tile
     auto body = [&](int vbuf, auto nb_tag, int cbuf, int cnb, int kbuf, int knb, auto &&copy) {
@@ -374,6 +375,7 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
       const auto NB = nb_tag;
       if (!QK_ONLY) v_frags(vbuf, NB, std::integral_constant<int, 0>{}, vr0);
       __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(1);
       // INT8 product of block b+1 under the exponentials of the first 16 keys of block b
 #pragma unroll
       for (int v = 0; v < 16; ++v) s[v] = 0;
@@ -382,6 +384,7 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
       float l0, l1;
       if (!QK_ONLY) exp_half(0, pf0, l0);
       __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(0);
       copy(std::integral_constant<int, 0>{});
       if (!QK_ONLY) {
         check_half(0, pf0, l0);
@@ -395,6 +398,7 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
         sk4[aa] = *reinterpret_cast<const f32x4 *>(cb + (32 * cnb + 8 * aa + 4 * g) * 4);
       const u32x4 corr_k = {reinterpret_cast<const unsigned *>(cb + FWD_BN * 4)[2 * (32 * cnb + lr) + g], 0u, 0u, 0u};
       __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(1);
       if (!QK_ONLY) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
@@ -403,6 +407,7 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
         exp_half(1, pf1, l1);
       }
       __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(0);
       if (!QK_ONLY) {
         check_half(1, pf1, l1);
         lds_wait_async<0>(vr1);   // everything requested so far was requested a phase ago
@@ -410,6 +415,7 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
       copy(std::integral_constant<int, 1>{});
       k_frags(kbuf, knb);
       __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(1);
       f32x16 f;
       if (!QK_ONLY) {
 #pragma unroll
@@ -428,6 +434,7 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
       copy(std::integral_constant<int, 2>{});
       f = mfma_16b<T>(corr_k, corr_q, f);
       __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(0);
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa)
 #pragma unroll
