@@ -33,7 +33,7 @@
 //  * row sums are taken over packed pairs with v_dot2;
 //  * tiles without any masked score run a software-pipelined loop whose body is one straight
 //    basic block per 32-key block: exp2/pack of block b, the P.V MFMAs of block b, the INT8 MFMAs
-//    of block b+2 and the convert/correct/scale/max of block b+1 are independent of each other,
+//    of block b+2 and the convert/correct/scale of block b+1 are independent of each other,
 //    so MFMA and VALU instructions interleave; diagonal and ragged tiles run a simple masked loop.
 //
 // V lies in LDS as it does in memory ([key][d] rows, 64-byte quarters XOR-swizzled against bank
@@ -310,7 +310,7 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
   int t = 0;
   if (t_hot > 0) {
     // ---- pipelined loop over unmasked tiles, one straight-line body per 32-key block b:
-    //   exp2/pack and P.V of block b | INT8 product of block b+1 | convert/correct/scale/max of b+1,
+    //   exp2/pack and P.V of block b | INT8 product of block b+1 | convert/correct/scale of b+1,
     // with every LDS operand requested a phase (or a body) before the MFMA that consumes it.  The
     // phases are fenced so that the requests stay where they are; inside a phase MFMA and VALU
     // instructions are independent and interleave.  A wave raises its issue priority for the phases that

@@ -91,3 +91,39 @@ def test_shared_kv_random_sweep(qfa):
         assert_close(case + " dQ", dq.cpu(), dq_ref, scaled=True, cos_tol=-1 if one_hot else 0.999)
         assert_close(case + " dKV", dkv.cpu(), dkv_ref, scaled=True)
         assert torch.isfinite(dq).all() and torch.isfinite(dkv).all(), case
+
+
+def test_backward_random_sweep(qfa):
+    """Forward + backward of the INT8-score kernels; head counts from 1 to 20 so that the causal dispatch
+    groups (2 to 8 heads) come out full, partial and absent."""
+    rng = random.Random(777)
+    for it in range(72):
+        D = rng.choice((64, 128))
+        dt = rng.choice((torch.bfloat16, torch.float16))
+        causal = rng.random() < 0.6
+        B, H = rng.choice(((1, 1), (1, 2), (2, 2), (3, 3), (2, 5), (1, 16), (4, 5)))
+        Nk = rng.choice((64, 128, 192, 256, 320, 384, 100, 333, 129, 65, 500))
+        Nq = Nk if causal else rng.choice((Nk, 128, 256, 97, 17))
+        kind = rng.choice(("normal", "ramp", "spike", "big"))
+        g = torch.Generator().manual_seed(5000 + it)
+        q = torch.randn((B, H, Nq, D), generator=g)
+        k = torch.randn((B, H, Nk, D), generator=g)
+        v = torch.randn((B, H, Nk, D), generator=g).to(dt)
+        do = torch.randn((B, H, Nq, D), generator=g).to(dt)
+        q, k = _scores(kind, q, k, Nk, g)
+        if kind == "big":
+            q, k = q * 0.5, k * (2.0 / 3.0)
+        q, k = q.to(dt), k.to(dt)
+        sm = 1.0 / math.sqrt(D)
+        qq, kq = qfa.quantize_for_attention(q.to(DEV)), qfa.quantize_for_attention(k.to(DEV))
+        o, lse = qfa.attn_fwd_quantized(qq, kq, v.to(DEV), causal, sm)
+        dq, dk, dv = qfa.attn_bwd_quantized(qq, kq, v.to(DEV), o, do.to(DEV), lse, causal, sm)
+        qh = oracle.dequantize_per_token(qq.codes.cpu(), qq.scale.cpu(), qq.zero_point.cpu(), torch.float64)
+        kh = oracle.dequantize_per_token(kq.codes.cpu(), kq.scale.cpu(), kq.zero_point.cpu(), torch.float64)
+        rq, rk, rv = oracle.attn_bwd(qh, kh, v, do, causal, sm)
+        case = f"case {it}: {kind} B{B} H{H} Nq{Nq} Nk{Nk} D{D} {dt} causal={causal}"
+        cos = 0.999 if kind == "normal" else -1   # nearly one-hot rows: the rounding of O alone moves small dQ, dK
+        assert_close(case + " dQ", dq.cpu(), rq, scaled=True, cos_tol=cos)
+        assert_close(case + " dK", dk.cpu(), rk, scaled=True, cos_tol=cos)
+        assert_close(case + " dV", dv.cpu(), rv, scaled=True, cos_tol=0.99)
+        assert torch.isfinite(dq).all() and torch.isfinite(dk).all() and torch.isfinite(dv).all(), case
