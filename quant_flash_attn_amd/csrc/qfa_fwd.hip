@@ -365,8 +365,8 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
     };
     // one body: V block (vbuf, nb); scores of the next block from kf; its constants in (cbuf, cnb);
     // then kf is refilled from K block (kbuf, knb).
-    // `copy(i)`, i = 0..2, is called between phases: the steady loop issues one chunk of the next
-    // tiles' copies there, so that the memory pipe sees single requests instead of a burst per tile
+    // `copy(i)`, i = 0..2, is called between phases: the steady loop issues chunks of the next
+    // tiles' copies there, so that the memory pipe sees a few requests at a time instead of a burst per tile
     auto body = [&](int vbuf, auto nb_tag, int cbuf, int cnb, int kbuf, int knb, auto &&copy) {
       static_assert(DB == 4 || DB == 2, "fragment arrays are sized for head_dim 128 or 64");
       u32x2 vr0[2 * DB], vr1[2 * DB];
@@ -451,8 +451,10 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
       k_frags(0, 1);
     }
     auto no_copy = [](auto) {};
-    // steady state: K(t+2) and V(t+1) are full tiles; their chunks (K first, then V) go out one at a
-    // time between the phases of the two bodies
+    // steady state: K(t+2) and V(t+1) are full tiles; their chunks (K first, then V) go out two at a
+    // time between the phases of the tile's first body, so that the last of them has the whole second body
+    // to land before the wait at the end of the tile (2 % at the causal headline size against one chunk
+    // per phase over both bodies; all six at once, or three and three, are slower again)
     for (; t < t_hot && t + 2 < ntiles && (t + 3) * FWD_BN <= a.Nk; ++t) {
       load_kc(t + 2);
       const rsrc_t rs_k =
@@ -465,8 +467,11 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
         if (i < KCH) cp_k.issue_one(rs_k, kd, wave_u, tid, i);
         else if (i < KCH + VCH) cp_v.issue_one(rs_v, vd, wave_u, tid, i - KCH);
       };
-      body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, [&](auto i) { chunk(decltype(i)::value); });
-      body(t & 1, std::integral_constant<int, 1>{}, kb_nxt, 0, kb_nxt, 1, [&](auto i) { chunk(3 + decltype(i)::value); });
+      body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, [&](auto i) {
+        chunk(2 * decltype(i)::value);
+        chunk(2 * decltype(i)::value + 1);
+      });
+      body(t & 1, std::integral_constant<int, 1>{}, kb_nxt, 0, kb_nxt, 1, no_copy);
       static_assert(KCH + VCH <= 6, "six copy slots per tile");
       store_k(kb_free);
       const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
