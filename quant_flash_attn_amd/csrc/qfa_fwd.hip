@@ -311,7 +311,9 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
   if (t_hot > 0) {
     // ---- pipelined loop over unmasked tiles, one straight-line body per 32-key block b:
     //   exp2/pack and P.V of block b | INT8 product of block b+1 | convert/correct/scale of b+1,
-    // with every LDS operand requested a phase (or a body) before the MFMA that consumes it.  The
+    // with every LDS operand requested a phase (or a body) before the MFMA that consumes it and every MFMA
+    // result read a phase after the MFMA was issued (the chain convert -> correction MFMA -> scale is spread
+    // over the two P.V phases).  The
     // phases are fenced so that the requests stay where they are; inside a phase MFMA and VALU
     // instructions are independent and interleave.  A wave raises its issue priority for the phases that
     // hold MFMAs and drops it for the ones that wait and request, so that of the two waves of a SIMD the
@@ -373,6 +375,11 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
       u32x4 pf0, pf1;
       i32x16 s;
       const auto NB = nb_tag;
+      // The K fragments were requested a body ago.  The compiler's counted wait for them must come HERE,
+      // before the V requests it does not know of: in front of the INT8 MFMAs it would cover those too
+      // (LDS returns in order) and the matrix pipe would idle for a full LDS round trip per block.
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(kf[ks]));
       if (!QK_ONLY) v_frags(vbuf, NB, std::integral_constant<int, 0>{}, vr0);
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(1);
@@ -398,30 +405,17 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
         sk4[aa] = *reinterpret_cast<const f32x4 *>(cb + (32 * cnb + 8 * aa + 4 * g) * 4);
       const u32x4 corr_k = {reinterpret_cast<const unsigned *>(cb + FWD_BN * 4)[2 * (32 * cnb + lr) + g], 0u, 0u, 0u};
       __builtin_amdgcn_sched_barrier(0);
+      // P.V of the first 16 keys under the exponentials of the second 16 and the conversion of the next
+      // block's raw scores; their zero-point correction (one MFMA) goes last, so that its result has the
+      // whole next phase to arrive before the scaling reads it
       __builtin_amdgcn_s_setprio(1);
+      f32x16 f;
       if (!QK_ONLY) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
           oacc[db] = mfma_16b<T>(u32x4{vr0[2 * db][0], vr0[2 * db][1], vr0[2 * db + 1][0], vr0[2 * db + 1][1]}, pf0,
                                  oacc[db]);
         exp_half(1, pf1, l1);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_setprio(0);
-      if (!QK_ONLY) {
-        check_half(1, pf1, l1);
-        lds_wait_async<0>(vr1);   // everything requested so far was requested a phase ago
-      }
-      copy(std::integral_constant<int, 1>{});
-      k_frags(kbuf, knb);
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_setprio(1);
-      f32x16 f;
-      if (!QK_ONLY) {
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-          oacc[db] = mfma_16b<T>(u32x4{vr1[2 * db][0], vr1[2 * db][1], vr1[2 * db + 1][0], vr1[2 * db + 1][1]}, pf1,
-                                 oacc[db]);
       } else {
         float sm = 0.f;
 #pragma unroll
@@ -431,14 +425,31 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
       __builtin_amdgcn_sched_barrier(0);
-      copy(std::integral_constant<int, 2>{});
       f = mfma_16b<T>(corr_k, corr_q, f);
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(0);
+      if (!QK_ONLY) {
+        check_half(1, pf1, l1);
+        lds_wait_async<0>(vr1);   // everything requested so far was requested a phase ago
+      }
+      copy(std::integral_constant<int, 1>{});
+      k_frags(kbuf, knb);
+      __builtin_amdgcn_sched_barrier(0);
+      // P.V of the second 16 keys under the scaling of the next block's scores
+      __builtin_amdgcn_s_setprio(1);
+      if (!QK_ONLY) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+          oacc[db] = mfma_16b<T>(u32x4{vr1[2 * db][0], vr1[2 * db][1], vr1[2 * db + 1][0], vr1[2 * db + 1][1]}, pf1,
+                                 oacc[db]);
+      }
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa)
 #pragma unroll
         for (int bb = 0; bb < 4; ++bb) u[4 * aa + bb] = f[4 * aa + bb] * sk4[aa][bb];
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(0);
+      copy(std::integral_constant<int, 2>{});
     };
 
     {   // block 0 prepared, fragments of block 1 in flight
