@@ -41,7 +41,7 @@ PEAK_HBM_GBS = 8000.0
 # FETCH_SIZE 195 063 KiB x 2.000 (calibration: 256 MiB copy reads 131 085) + WRITE_SIZE 133 195 KiB x 1.000
 # (profiles/kernels_B4_H32_N4096_D128_causal_bf16.md); algorithmic bytes are 395 MiB -- the causal dispatch
 # order keeps four heads in flight per XCD, more than its L2 holds, and the re-reads show up here
-FWD_TRAFFIC_BYTES = (195063 * 2 + 133195) * 1024
+FWD_TRAFFIC_BYTES = (193050 * 2 + 133233) * 1024
 
 
 def flops_fwd(B, H, Nq, Nk, D, causal):
