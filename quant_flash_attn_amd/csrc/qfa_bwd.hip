@@ -451,7 +451,8 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(BwdArgs a) {
 // One workgroup = 128 keys = 8 waves.  The dK^T and dV^T accumulators of 32 keys take 128 registers,
 // too many for two waves per SIMD, so each 32-key slice is shared by a PAIR of waves that sit on the
 // same SIMD (waves w and w+4):
-//   P-wave  (w < 4):  S = Qc.Kc^T (INT8 MFMA), P = exp2(.), hands P to its partner through LDS,
+//   P-wave  (w < 4):  S = Qc.Kc^T (INT8 MFMA), P = exp2(.), hands P to its partner through LDS (rounded to
+//                     the 16-bit type, as its own dV product uses it: half the exchange traffic of fp32),
 //                     dV^T += dO^T.P
 //   dS-wave (w >= 4): dP = dO.V^T, then dS' = P o (dP - delta) * a with the partner's P,
 //                     dK^T += Qz^T.dS'
@@ -460,6 +461,18 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(BwdArgs a) {
 // to the exchange slot of the block's parity, so the slot written for block b is read before barrier
 // b+1 and not written again before that barrier has passed.
 constexpr int DKV_THREADS = 512;
+
+// two 16-bit floats of one dword -> fp32
+template <typename T> __device__ __forceinline__ float unpack_lo(unsigned w);
+template <typename T> __device__ __forceinline__ float unpack_hi(unsigned w);
+template <> __device__ __forceinline__ float unpack_lo<__bf16>(unsigned w) { return __builtin_bit_cast(float, w << 16); }
+template <> __device__ __forceinline__ float unpack_hi<__bf16>(unsigned w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+template <> __device__ __forceinline__ float unpack_lo<_Float16>(unsigned w) {
+  return (float)__builtin_bit_cast(_Float16, (unsigned short)(w & 0xffffu));
+}
+template <> __device__ __forceinline__ float unpack_hi<_Float16>(unsigned w) {
+  return (float)__builtin_bit_cast(_Float16, (unsigned short)(w >> 16));
+}
 
 template <typename T, int D, bool CAUSAL>
 __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
@@ -471,8 +484,8 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
   constexpr int Q_BYTES = BWD_TILE * D, G_BYTES = BWD_TILE * 2 * D, T_BYTES = WS::T_BYTES;
   constexpr int OFF_DO = Q_BYTES, OFF_DOT = OFF_DO + G_BYTES, OFF_QT = OFF_DOT + T_BYTES, OFF_C = OFF_QT + T_BYTES,
                 BUF = OFF_C + WS::CQ_BYTES;
-  constexpr int OFF_X = 2 * BUF;             // P exchange: 2 slots x 4 pairs x 64 lanes x 16 floats
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF + 2 * 4 * 4096];
+  constexpr int OFF_X = 2 * BUF;             // P exchange: per pair 2 slots x 64 lanes x 16 packed 16-bit floats
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF + 4 * 4096];
 
   const int L = blockIdx.x;
   const int vid = (L % 8) * a.blocks_per_xcd + (L / 8);
@@ -567,9 +580,9 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) oacc[db][v] = 0.f;
 
-  // [slot][4][64 lanes] of 4 floats; the slot is the block's parity, so that one barrier per block is
+  // [slot][2][64 lanes] of 8 packed 16-bit floats; the slot is the block's parity, so that one barrier per block is
   // enough: P(b) is written before barrier b and read before barrier b+1, P(b+2) is written after it
-  f32x4 *xch0 = reinterpret_cast<f32x4 *>(smem + OFF_X + pair * 4096);
+  u32x4 *xch0 = reinterpret_cast<u32x4 *>(smem + OFF_X + pair * 4096);
 
   // LDS operands are fetched in groups well ahead of the MFMAs that consume them (a 16-byte LDS read
   // takes far longer than an MFMA issue slot, and the compiler keeps loads next to their use), the
@@ -606,7 +619,6 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
 #pragma unroll
     for (int aa = 0; aa < 4; ++aa) {
       const int il = 32 * mbk + 8 * aa + 4 * g;
-      f32x4 p4;
 #pragma unroll
       for (int bb = 0; bb < 4; ++bb) {
         float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a4[aa][bb], f[4 * aa + bb] * sk_j, nl4[aa][bb]));
@@ -615,14 +627,14 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
           if ((CAUSAL && kj > i) || i >= a.Nq || kj >= a.Nk) p = 0.f;
         }
         pp[4 * aa + bb] = p;
-        p4[bb] = p;
       }
-      xch0[mbk * 1024 + aa * 64 + lane] = p4;
     }
 #pragma unroll
-    for (int hh = 0; hh < 2; ++hh)
+    for (int hh = 0; hh < 2; ++hh) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) pf[hh][e] = pack2<T>(pp[8 * hh + 2 * e], pp[8 * hh + 2 * e + 1]);
+      xch0[mbk * 128 + hh * 64 + lane] = pf[hh];
+    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh)
@@ -663,14 +675,18 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
   };
   // ---- dS role, second half prologue: dS' = P (from partner) * (dP - delta) * a, packed
   auto ds_second = [&](int mbk, const f32x16 &dp, const f32x4 (&a4)[4], const f32x4 (&dl4)[4], u32x4 (&dsf)[2]) {
-    f32x4 p4[4];
+    u32x4 pw[2];
 #pragma unroll
-    for (int aa = 0; aa < 4; ++aa) p4[aa] = xch0[mbk * 1024 + aa * 64 + lane];
+    for (int hh = 0; hh < 2; ++hh) pw[hh] = xch0[mbk * 128 + hh * 64 + lane];
     float ds[16];
 #pragma unroll
-    for (int aa = 0; aa < 4; ++aa)
+    for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
-      for (int bb = 0; bb < 4; ++bb) ds[4 * aa + bb] = p4[aa][bb] * (dp[4 * aa + bb] - dl4[aa][bb]) * a4[aa][bb];
+      for (int e = 0; e < 4; ++e) {
+        const int v = 8 * hh + 2 * e;
+        ds[v] = unpack_lo<T>(pw[hh][e]) * (dp[v] - dl4[v / 4][v % 4]) * a4[v / 4][v % 4];
+        ds[v + 1] = unpack_hi<T>(pw[hh][e]) * (dp[v + 1] - dl4[(v + 1) / 4][(v + 1) % 4]) * a4[(v + 1) / 4][(v + 1) % 4];
+      }
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
