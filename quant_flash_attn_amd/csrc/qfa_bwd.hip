@@ -1,7 +1,7 @@
 // Backward kernels for gfx950: two staging passes, then two MFMA kernels that recompute
 // P = exp(S - LSE) from the INT8 codes exactly as the forward does.
 //
-//   prep_q       per 64-query tile: delta = rowsum(O o dO) in fp32; dO^T and Qz^T = (Qc - zq)^T as
+//   prep_q       per 64-query tile: delta = rowsum(O o dO) in fp32; dO^T and Qz^T = ((Qc - zq) * sq)^T as
 //                16-bit tiles [d][query] in the key order the MFMA layouts want; per-query constants
 //   prep_k       per 64-key tile: Kz^T = (Kc - zk)^T likewise; per-key constants
 //                (both write into the caller's workspace; every tile is converted and transposed
@@ -11,14 +11,17 @@
 //                dQ^T += Kz^T.(dS^T * sk)         with Kz = (Kc - zk) held as exact 16-bit floats
 //   dkdv kernel  one workgroup = 128 keys (32 per wave), loops over 64-query tiles.
 //                S = Qc.Kc^T (INT8 MFMA), dP = dO.V^T, dV^T += dO^T.P,
-//                dK^T += Qz^T.(dS * sq)           with Qz = (Qc - zq)
+//                dK^T += Qz^T.dS                  with Qz = (Qc - zq) * sq, the dequantized Q rounded to 16 bits
 // In both, the wave's own operand (queries resp. keys) stays in registers as the MFMA B operand
 // for the whole loop and the streamed operand comes from LDS as the A operand.  The 32x32
 // accumulator layout then leaves P / dS in registers exactly in the B-operand layout of the next
 // product; the transposed LDS tiles (Kz^T, dO^T, Qz^T) are written in the matching permuted order.
 // dQ is produced by its own kernel instead of atomics, so results are deterministic.
-// (Kc - zk) and (Qc - zq) are integers in [-255, 255]: exact in bf16 and fp16, so the scales are
-// folded into dS in fp32 and dequantization adds no rounding error.
+// (Kc - zk) is an integer in [-255, 255]: exact in bf16 and fp16, so in the dQ kernel the key scale is
+// folded into dS in fp32 and dequantization adds no rounding error.  The dK/dV kernel is bound by LDS reads
+// (48 KB per 32x32 block and wave pair, of which the per-query constants were 16 KB), so there the query
+// scale is folded into the Qz^T tile instead, which takes one constant vector out of the loop: Qz is then
+// the dequantized Q rounded to the 16-bit type, the operand an unquantized backward would use.
 #include <type_traits>
 
 #include "qfa_device.h"
@@ -126,13 +129,13 @@ __device__ __forceinline__ int perm_pos4(int r4) {   // r4 = r / 4
 // (code - zp) for the 8 codes in two dwords of 4 rows, as exact 16-bit floats, transposed:
 // writes, for each of the 8 columns, the 4 rows as 8 bytes at dst + column * stride
 template <typename T>
-__device__ __forceinline__ void store_codes_transposed(const u32x2 (&c)[4], const float (&zp)[4], unsigned char *dst,
-                                                       int stride) {
+__device__ __forceinline__ void store_codes_transposed(const u32x2 (&c)[4], const float (&zp)[4], const float (&sc)[4],
+                                                       unsigned char *dst, int stride) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     float f[4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) f[r] = (float)(int)(int8_t)((c[r][e / 4] >> (8 * (e % 4))) & 0xff) - zp[r];
+    for (int r = 0; r < 4; ++r) f[r] = ((float)(int)(int8_t)((c[r][e / 4] >> (8 * (e % 4))) & 0xff) - zp[r]) * sc[r];
     u32x2 o;
     o[0] = pack2<T>(f[0], f[1]);
     o[1] = pack2<T>(f[2], f[3]);
@@ -179,7 +182,7 @@ template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_q_k
     const T *o_bh = reinterpret_cast<const T *>(a.o) + b * a.sob + h * a.soh;
     u32x2 creg[4];
     u32x4 greg[4];
-    float zreg[4];
+    float zreg[4], sreg[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int i = min(i0 + 4 * r4 + r, a.Nq - 1);
@@ -187,6 +190,7 @@ template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_q_k
       greg[r] = *reinterpret_cast<const u32x4 *>(do_bh + (int64_t)i * a.sdon + dc * 8);
       const u32x4 ow = *reinterpret_cast<const u32x4 *>(o_bh + (int64_t)i * a.son + dc * 8);
       zreg[r] = (float)a.zq[tq0 + i];
+      sreg[r] = a.sq[tq0 + i];
       float s = 0.f;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -197,7 +201,8 @@ template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_q_k
     }
     const int pos = perm_pos4(r4);
     store_16b_transposed(greg, blob + (dc * 8) * (BWD_TILE * 2) + pos * 2, BWD_TILE * 2);
-    store_codes_transposed<T>(creg, zreg, blob + WS::T_BYTES + (dc * 8) * (BWD_TILE * 2) + pos * 2, BWD_TILE * 2);
+    // the dequantized Q itself, rounded to the 16-bit type (what dK = sm * dS^T Q^ contracts with)
+    store_codes_transposed<T>(creg, zreg, sreg, blob + WS::T_BYTES + (dc * 8) * (BWD_TILE * 2) + pos * 2, BWD_TILE * 2);
   }
   __syncthreads();
   if (tid < BWD_TILE) {
@@ -238,7 +243,8 @@ template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_k_k
       creg[r] = *reinterpret_cast<const u32x2 *>(kc_bh + (int64_t)j * a.skn + dc * 8);
       zreg[r] = (float)a.zk[tk0 + j];
     }
-    store_codes_transposed<T>(creg, zreg, blob + (dc * 8) * (BWD_TILE * 2) + perm_pos4(r4) * 2, BWD_TILE * 2);
+    const float ones[4] = {1.f, 1.f, 1.f, 1.f};
+    store_codes_transposed<T>(creg, zreg, ones, blob + (dc * 8) * (BWD_TILE * 2) + perm_pos4(r4) * 2, BWD_TILE * 2);
   }
   if (tid < BWD_TILE) {
     const int j = min(j0 + tid, a.Nk - 1);
@@ -454,8 +460,8 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(BwdArgs a) {
 //   P-wave  (w < 4):  S = Qc.Kc^T (INT8 MFMA), P = exp2(.), hands P to its partner through LDS (rounded to
 //                     the 16-bit type, as its own dV product uses it: half the exchange traffic of fp32),
 //                     dV^T += dO^T.P
-//   dS-wave (w >= 4): dP = dO.V^T, then dS' = P o (dP - delta) * a with the partner's P,
-//                     dK^T += Qz^T.dS'
+//   dS-wave (w >= 4): dP = dO.V^T, then dS = P o (dP - delta) with the partner's P,
+//                     dK^T += Qz^T.dS
 // No product is computed twice, each wave keeps 64 accumulator registers, and within a SIMD one wave
 // is in its VALU phase while the other feeds the matrix pipe.  One barrier per 32-query block: P goes
 // to the exchange slot of the block's parity, so the slot written for block b is read before barrier
@@ -643,7 +649,7 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
         tf[hh * DB + db] = *reinterpret_cast<const u32x4 *>(base + OFF_DOT + ST::off(32 * db + lr, 4 * mbk + 2 * hh + g));
   };
   // ---- dS role, first half: dP = dO.V^T; then the Qz^T fragments and constants of the second half
-  auto ds_first = [&](const unsigned char *base, int mbk, f32x16 &dp, u32x4 (&tf)[2 * DB], f32x4 (&a4)[4], f32x4 (&dl4)[4]) {
+  auto ds_first = [&](const unsigned char *base, int mbk, f32x16 &dp, u32x4 (&tf)[2 * DB], f32x4 (&dl4)[4]) {
     const float *cs = reinterpret_cast<const float *>(base + OFF_C);
     u32x4 gf[KD];
 #pragma unroll
@@ -662,7 +668,6 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
 #pragma unroll
     for (int aa = 0; aa < 4; ++aa) {
       const int il = 32 * mbk + 8 * aa + 4 * g;
-      a4[aa] = *reinterpret_cast<const f32x4 *>(cs + 2 * BWD_TILE + il);
       dl4[aa] = *reinterpret_cast<const f32x4 *>(cs + 4 * BWD_TILE + il);
     }
   };
@@ -673,8 +678,8 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
 #pragma unroll
       for (int db = 0; db < DB; ++db) oacc[db] = mfma_16b<T>(tf[hh * DB + db], bf[hh], oacc[db]);
   };
-  // ---- dS role, second half prologue: dS' = P (from partner) * (dP - delta) * a, packed
-  auto ds_second = [&](int mbk, const f32x16 &dp, const f32x4 (&a4)[4], const f32x4 (&dl4)[4], u32x4 (&dsf)[2]) {
+  // ---- dS role, second half prologue: dS = P (from partner) * (dP - delta), packed
+  auto ds_second = [&](int mbk, const f32x16 &dp, const f32x4 (&dl4)[4], u32x4 (&dsf)[2]) {
     u32x4 pw[2];
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh) pw[hh] = xch0[mbk * 128 + hh * 64 + lane];
@@ -684,8 +689,8 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int v = 8 * hh + 2 * e;
-        ds[v] = unpack_lo<T>(pw[hh][e]) * (dp[v] - dl4[v / 4][v % 4]) * a4[v / 4][v % 4];
-        ds[v + 1] = unpack_hi<T>(pw[hh][e]) * (dp[v + 1] - dl4[(v + 1) / 4][(v + 1) % 4]) * a4[(v + 1) / 4][(v + 1) % 4];
+        ds[v] = unpack_lo<T>(pw[hh][e]) * (dp[v] - dl4[v / 4][v % 4]);
+        ds[v + 1] = unpack_hi<T>(pw[hh][e]) * (dp[v + 1] - dl4[(v + 1) / 4][(v + 1) % 4]);
       }
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh)
@@ -743,8 +748,8 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
         block_flags(t, mbk, on, masked);
         u32x4 dsf[2], tf[2 * DB];
         f32x16 dp;
-        f32x4 a4[4], dl4[4];
-        if (on) ds_first(base, mbk, dp, tf, a4, dl4);
+        f32x4 dl4[4];
+        if (on) ds_first(base, mbk, dp, tf, dl4);
         if (mbk == 1) dma_wait();
         lds_barrier();
         if (mbk == 0 && t + 1 < ntiles) {
@@ -752,7 +757,7 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
           load_part(t + 1, 3);
         }
         if (on) {
-          ds_second(mbk, dp, a4, dl4, dsf);
+          ds_second(mbk, dp, dl4, dsf);
           accumulate(tf, dsf);
         }
       }
@@ -761,7 +766,7 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
 
   if (kj < a.Nk) {
     T *row = (p_role ? dv_bh + (int64_t)kj * a.sdvn : dk_bh + (int64_t)kj * a.sdkn);
-    const float scale = p_role ? 1.0f : kLn2;
+    const float scale = p_role ? 1.0f : a.sm_scale;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
