@@ -3,12 +3,12 @@
 //
 //   prep_q       per 64-query tile: delta = rowsum(O o dO) in fp32; dO^T and Qz^T = ((Qc - zq) * sq)^T as
 //                16-bit tiles [d][query] in the key order the MFMA layouts want; per-query constants
-//   prep_k       per 64-key tile: Kz^T = (Kc - zk)^T likewise; per-key constants
+//   prep_k       per 64-key tile: Kz^T = ((Kc - zk) * sk)^T likewise; per-key constants
 //                (both write into the caller's workspace; every tile is converted and transposed
 //                once instead of once per consuming workgroup)
 //   dq kernel    one workgroup = 128 queries (32 per wave), loops over 64-key tiles.
 //                S^T = Kc.Qc^T (INT8 MFMA), dP^T = V.dO^T, dS^T = P^T o (dP^T - delta),
-//                dQ^T += Kz^T.(dS^T * sk)         with Kz = (Kc - zk) held as exact 16-bit floats
+//                dQ^T += Kz^T.dS^T                with Kz = (Kc - zk) * sk, the dequantized K rounded to 16 bits
 //   dkdv kernel  one workgroup = 128 keys (32 per wave), loops over 64-query tiles.
 //                S = Qc.Kc^T (INT8 MFMA), dP = dO.V^T, dV^T += dO^T.P,
 //                dK^T += Qz^T.dS                  with Qz = (Qc - zq) * sq, the dequantized Q rounded to 16 bits
@@ -17,11 +17,10 @@
 // accumulator layout then leaves P / dS in registers exactly in the B-operand layout of the next
 // product; the transposed LDS tiles (Kz^T, dO^T, Qz^T) are written in the matching permuted order.
 // dQ is produced by its own kernel instead of atomics, so results are deterministic.
-// (Kc - zk) is an integer in [-255, 255]: exact in bf16 and fp16, so in the dQ kernel the key scale is
-// folded into dS in fp32 and dequantization adds no rounding error.  The dK/dV kernel is bound by LDS reads
-// (48 KB per 32x32 block and wave pair, of which the per-query constants were 16 KB), so there the query
-// scale is folded into the Qz^T tile instead, which takes one constant vector out of the loop: Qz is then
-// the dequantized Q rounded to the 16-bit type, the operand an unquantized backward would use.
+// The scales of the streamed operand are folded into its transposed 16-bit tile (Kz^T, Qz^T) by the staging
+// pass, so dS is used as it comes: the tiles then hold the dequantized K and Q rounded to the 16-bit type, the
+// operands an unquantized backward would use.  The dK/dV kernel is bound by LDS reads (48 KB per 32x32 block
+// and wave pair, 16 KB of it per-query constants), and the fold takes one constant vector out of its loop.
 #include <type_traits>
 
 #include "qfa_device.h"
@@ -236,15 +235,16 @@ template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_k_k
   if (dc < D / 8) {
     const int8_t *kc_bh = a.kc + b * a.skb + h * a.skh;
     u32x2 creg[4];
-    float zreg[4];
+    float zreg[4], sreg[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int j = min(j0 + 4 * r4 + r, a.Nk - 1);
       creg[r] = *reinterpret_cast<const u32x2 *>(kc_bh + (int64_t)j * a.skn + dc * 8);
       zreg[r] = (float)a.zk[tk0 + j];
+      sreg[r] = a.sk[tk0 + j];
     }
-    const float ones[4] = {1.f, 1.f, 1.f, 1.f};
-    store_codes_transposed<T>(creg, zreg, ones, blob + (dc * 8) * (BWD_TILE * 2) + perm_pos4(r4) * 2, BWD_TILE * 2);
+    // the dequantized K, rounded to the 16-bit type (what dQ = sm * dS K^ contracts with)
+    store_codes_transposed<T>(creg, zreg, sreg, blob + (dc * 8) * (BWD_TILE * 2) + perm_pos4(r4) * 2, BWD_TILE * 2);
   }
   if (tid < BWD_TILE) {
     const int j = min(j0 + tid, a.Nk - 1);
@@ -403,7 +403,7 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(BwdArgs a) {
           const int j = j0 + jl + bb;
           if ((CAUSAL && j > qi) || j >= a.Nk) p = 0.f;
         }
-        ds[v] = p * (dp[v] - delta_i) * sk4[bb];
+        ds[v] = p * (dp[v] - delta_i);
       }
     }
 #pragma unroll
