@@ -82,7 +82,6 @@ int launch_delta(const void *o, const void *dout, float *delta, int io_dtype, in
 }
 
 // ------------------------------------------------------------------------------------------ shared
-constexpr int BWD_BLK = 128;   // rows owned by a workgroup
 constexpr int BWD_TILE = 64;   // rows streamed per step
 
 // Workspace layout: per (batch*head, 64-query tile) a Q-side blob, then per (batch*head, 64-key tile)
@@ -462,19 +461,28 @@ __global__ __launch_bounds__(DqShape<D>::THREADS, DqShape<D>::WAVES_PER_SIMD) vo
 }
 
 // ------------------------------------------------------------------------------------------ dK, dV
-// One workgroup = 128 keys = 8 waves.  The dK^T and dV^T accumulators of 32 keys take 128 registers,
-// too many for two waves per SIMD, so each 32-key slice is shared by a PAIR of waves that sit on the
-// same SIMD (waves w and w+4):
-//   P-wave  (w < 4):  S = Qc.Kc^T (INT8 MFMA), P = exp2(.), hands P to its partner through LDS (rounded to
+// One workgroup = 4 (head_dim 128) or 6 (head_dim 64) wave pairs of 32 keys each.  The dK^T and dV^T
+// accumulators of 32 keys take 128 registers at head_dim 128, too many for two waves per SIMD, so each 32-key
+// slice is shared by a PAIR of waves (w and w + pairs; with 4 pairs they sit on the same SIMD):
+//   P-wave  (w < pairs):  S = Qc.Kc^T (INT8 MFMA), P = exp2(.), hands P to its partner through LDS (rounded to
 //                     the 16-bit type, as its own dV product uses it: half the exchange traffic of fp32),
 //                     dV^T += dO^T.P
-//   dS-wave (w >= 4): dP = dO.V^T, then dS = P o (dP - delta) with the partner's P,
+//   dS-wave (the others): dP = dO.V^T, then dS = P o (dP - delta) with the partner's P,
 //                     dK^T += Qz^T.dS
 // No product is computed twice, each wave keeps 64 accumulator registers, and within a SIMD one wave
 // is in its VALU phase while the other feeds the matrix pipe.  One barrier per 32-query block: P goes
 // to the exchange slot of the block's parity, so the slot written for block b is read before barrier
 // b+1 and not written again before that barrier has passed.
-constexpr int DKV_THREADS = 512;
+// Wave pairs per workgroup (32 keys per pair) and waves per SIMD the registers are budgeted for.  One
+// workgroup runs per CU (the two tile buffers and the exchange fill the LDS).  D=128: 4 pairs, 2 waves per
+// SIMD (the loop takes 220 registers).  D=64: 6 pairs, 3 waves per SIMD (145 registers); backward of
+// B16 H16 N2048 D64 causal 0.84 -> 0.805 ms against 4 pairs; 3 pairs with two workgroups per CU are slower
+// (0.95 ms), 8 pairs need 128 registers and spill.
+template <int D> struct DkvShape {
+  static constexpr int PAIRS = D == 64 ? 6 : 4;
+  static constexpr int WAVES_PER_SIMD = D == 64 ? 3 : 2;
+  static constexpr int THREADS = 128 * PAIRS, BLK = 32 * PAIRS;
+};
 
 // two 16-bit floats of one dword -> fp32
 template <typename T> __device__ __forceinline__ float unpack_lo(unsigned w);
@@ -489,7 +497,8 @@ template <> __device__ __forceinline__ float unpack_hi<_Float16>(unsigned w) {
 }
 
 template <typename T, int D, bool CAUSAL>
-__global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
+__global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) void bwd_dkdv_kernel(BwdArgs a) {
+  constexpr int NP = DkvShape<D>::PAIRS, DKV_THREADS = DkvShape<D>::THREADS;
   typedef BwdWs<D> WS;
   typedef Swz<D> SQ;            // Q code rows
   typedef Swz<2 * D> SG;        // dO rows
@@ -499,7 +508,7 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
   constexpr int OFF_DO = Q_BYTES, OFF_DOT = OFF_DO + G_BYTES, OFF_QT = OFF_DOT + T_BYTES, OFF_C = OFF_QT + T_BYTES,
                 BUF = OFF_C + WS::CQ_BYTES;
   constexpr int OFF_X = 2 * BUF;             // P exchange: per pair 2 slots x 64 lanes x 16 packed 16-bit floats
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF + 4 * 4096];
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF + NP * 4096];
 
   const int L = blockIdx.x;
   const int vid = (L % 8) * a.blocks_per_xcd + (L / 8);
@@ -518,10 +527,10 @@ __global__ __launch_bounds__(DKV_THREADS, 2) void bwd_dkdv_kernel(BwdArgs a) {
     }
   }
   const int64_t b = bh / a.H, h = bh % a.H;
-  const int n0 = nbk * BWD_BLK;
+  const int n0 = nbk * DkvShape<D>::BLK;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, lr = lane % 32, g = lane / 32;
-  const int pair = wave % 4;
-  const bool p_role = wave < 4;      // wave-uniform
+  const int pair = wave % NP;
+  const bool p_role = wave < NP;     // wave-uniform
 
   const unsigned char *qc_bh = reinterpret_cast<const unsigned char *>(a.qc + b * a.sqb + h * a.sqh);
   const int8_t *kc_bh = a.kc + b * a.skb + h * a.skh;
@@ -814,7 +823,8 @@ template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStre
   if (int e = check_launch("qfa_attn_bwd (prep k)")) return e;
   // dK, dV
   {
-    a.nblocks = (int)((x.Nk + BWD_BLK - 1) / BWD_BLK);
+    constexpr int DKV_THREADS = DkvShape<D>::THREADS;
+    a.nblocks = (int)((x.Nk + DkvShape<D>::BLK - 1) / DkvShape<D>::BLK);
     // per head the kernel streams Qc, dO, dO^T and Qz^T (7 bytes per query and d): group heads while that
     // stays within an XCD's 4 MB L2 (one head already fills it at N=4096, D=128)
     const int64_t head_bytes = x.Nq * (int64_t)D * 7;
