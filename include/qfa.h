@@ -180,8 +180,10 @@ int qfa_bwd_delta(const void *o, const void *dout, float *delta, int io_dtype, i
  * kernel, :207-237 wrapper); the reference's single dKV tensor is dK + dV (:161).
  *   workspace  caller-owned scratch of at least qfa_attn_bwd_workspace_bytes(B,H,Nq,Nk,D) bytes,
  *              16-byte aligned, overwritten: two staging passes fill it with delta = rowsum(O o dO),
- *              the transposed 16-bit tiles dO^T, (Qc-zq)^T, (Kc-zk)^T and per-token constants, once
- *              per call, so that the two MFMA kernels stream ready-made tiles.
+ *              the transposed 16-bit tiles dO^T, Q^^T, K^^T (the dequantized Q and K rounded to
+ *              io_dtype, the operands of the dK and dQ products) and per-token constants, once
+ *              per call, so that the two MFMA kernels stream ready-made tiles.  The scores S, and
+ *              with them P, come from the INT8 codes exactly as in the forward.
  *   dq [B,H,Nq,D], dk, dv [B,H,Nk,D] of io_dtype, strides as given.
  */
 int64_t qfa_attn_bwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D);
