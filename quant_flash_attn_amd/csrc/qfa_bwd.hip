@@ -88,7 +88,7 @@ constexpr int BWD_TILE = 64;   // rows streamed per step
 // a K-side blob.  Transposed tiles are [D][64] 16-bit values, 128-byte rows, positions permuted.
 template <int D> struct BwdWs {
   static constexpr int T_BYTES = D * BWD_TILE * 2;            // one transposed tile
-  static constexpr int CQ_BYTES = 5 * BWD_TILE * 4;           // digits (2 dwords/query), a, -lse*log2e, delta
+  static constexpr int CQ_BYTES = 5 * BWD_TILE * 4;           // digits (2 dwords/query), a, -lse*log2e, -delta
   static constexpr int CK_BYTES = 3 * BWD_TILE * 4;           // digits (2 dwords/key), key scale
   static constexpr int Q_BLOB = 2 * T_BYTES + CQ_BYTES;       // dO^T, Qz^T, constants
   static constexpr int K_BLOB = T_BYTES + CK_BYTES;           // Kz^T, constants
@@ -217,7 +217,7 @@ template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_q_k
     reinterpret_cast<u32x2 *>(cq)[tid] = dg;
     reinterpret_cast<float *>(cq)[2 * BWD_TILE + tid] = a.sq[tq0 + i] * a.sm_scale_log2;
     reinterpret_cast<float *>(cq)[3 * BWD_TILE + tid] = -a.lse[tq0 + i] * kLog2e;
-    reinterpret_cast<float *>(cq)[4 * BWD_TILE + tid] = delta;
+    reinterpret_cast<float *>(cq)[4 * BWD_TILE + tid] = -delta;   // the dP accumulators start from it
   }
 }
 
@@ -319,13 +319,13 @@ __global__ __launch_bounds__(DqShape<D>::THREADS, DqShape<D>::WAVES_PER_SIMD) vo
 #pragma unroll
   for (int kd = 0; kd < KD; ++kd)
     dof[kd] = *reinterpret_cast<const u32x4 *>(do_bh + (int64_t)qi_c * a.sdon + kd * 16 + g * 8);
-  // per-query constants prepared by prep_q: correction digits, a = sq*sm*log2e, -lse*log2e, delta
+  // per-query constants prepared by prep_q: correction digits, a = sq*sm*log2e, -lse*log2e, -delta
   const unsigned *cq = reinterpret_cast<const unsigned *>(wsq_bh + (int64_t)(qi_c / BWD_TILE) * WS::Q_BLOB + 2 * WS::T_BYTES);
   const int ql = qi_c % BWD_TILE;
   const u32x4 corr_q = {cq[2 * ql + g], 0u, 0u, 0u};
   const float a_i = __builtin_bit_cast(float, cq[2 * BWD_TILE + ql]);
   const float nlse2 = __builtin_bit_cast(float, cq[3 * BWD_TILE + ql]);
-  const float delta_i = __builtin_bit_cast(float, cq[4 * BWD_TILE + ql]);
+  const float ndelta_i = __builtin_bit_cast(float, cq[4 * BWD_TILE + ql]);   // -delta
   const int q_first = m0 + wave * 32, q_last = q_first + 31;
 
   int kv_end = a.Nk;
@@ -381,7 +381,7 @@ __global__ __launch_bounds__(DqShape<D>::THREADS, DqShape<D>::WAVES_PER_SIMD) vo
     i32x16 acc;
     f32x16 dp;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) { acc[v] = 0; dp[v] = 0.f; }
+    for (int v = 0; v < 16; ++v) { acc[v] = 0; dp[v] = ndelta_i; }   // dp = dP^T - delta straight from the MFMAs
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const i32x4 kf = *reinterpret_cast<const i32x4 *>(base + SK::off(32 * nb + lr, 2 * ks + g));
@@ -410,7 +410,7 @@ __global__ __launch_bounds__(DqShape<D>::THREADS, DqShape<D>::WAVES_PER_SIMD) vo
           const int j = j0 + jl + bb;
           if ((CAUSAL && j > qi) || j >= a.Nk) p = 0.f;
         }
-        ds[v] = p * (dp[v] - delta_i);
+        ds[v] = p * dp[v];
       }
     }
 #pragma unroll
@@ -666,15 +666,20 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
         tf[hh * DB + db] = *reinterpret_cast<const u32x4 *>(base + OFF_DOT + ST::off(32 * db + lr, 4 * mbk + 2 * hh + g));
   };
   // ---- dS role, first half: dP = dO.V^T; then the Qz^T fragments and constants of the second half
-  auto ds_first = [&](const unsigned char *base, int mbk, f32x16 &dp, u32x4 (&tf)[2 * DB], f32x4 (&dl4)[4]) {
+  auto ds_first = [&](const unsigned char *base, int mbk, f32x16 &dp, u32x4 (&tf)[2 * DB]) {
     const float *cs = reinterpret_cast<const float *>(base + OFF_C);
     u32x4 gf[KD];
+    // the accumulators start from -delta of their rows, so that the MFMAs leave dP - delta
+#pragma unroll
+    for (int aa = 0; aa < 4; ++aa) {
+      const f32x4 nd = *reinterpret_cast<const f32x4 *>(cs + 4 * BWD_TILE + 32 * mbk + 8 * aa + 4 * g);
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) dp[4 * aa + bb] = nd[bb];
+    }
 #pragma unroll
     for (int kd = 0; kd < KD; ++kd)
       gf[kd] = *reinterpret_cast<const u32x4 *>(base + OFF_DO + SG::off(32 * mbk + lr, 2 * kd + g));
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int v = 0; v < 16; ++v) dp[v] = 0.f;
 #pragma unroll
     for (int kd = 0; kd < KD; ++kd) dp = mfma_16b<T>(gf[kd], breg[kd], dp);
 #pragma unroll
@@ -682,11 +687,6 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
 #pragma unroll
       for (int db = 0; db < DB; ++db)
         tf[hh * DB + db] = *reinterpret_cast<const u32x4 *>(base + OFF_QT + ST::off(32 * db + lr, 4 * mbk + 2 * hh + g));
-#pragma unroll
-    for (int aa = 0; aa < 4; ++aa) {
-      const int il = 32 * mbk + 8 * aa + 4 * g;
-      dl4[aa] = *reinterpret_cast<const f32x4 *>(cs + 4 * BWD_TILE + il);
-    }
   };
   // ---- second half: accumulate with the prefetched transposed fragments
   auto accumulate = [&](const u32x4 (&tf)[2 * DB], const u32x4 (&bf)[2]) {
@@ -695,8 +695,8 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
 #pragma unroll
       for (int db = 0; db < DB; ++db) oacc[db] = mfma_16b<T>(tf[hh * DB + db], bf[hh], oacc[db]);
   };
-  // ---- dS role, second half prologue: dS = P (from partner) * (dP - delta), packed
-  auto ds_second = [&](int mbk, const f32x16 &dp, const f32x4 (&dl4)[4], u32x4 (&dsf)[2]) {
+  // ---- dS role, second half prologue: dS = P (from partner) * (dP - delta), packed (dp holds dP - delta)
+  auto ds_second = [&](int mbk, const f32x16 &dp, u32x4 (&dsf)[2]) {
     u32x4 pw[2];
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh) pw[hh] = xch0[mbk * 128 + hh * 64 + lane];
@@ -706,8 +706,8 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int v = 8 * hh + 2 * e;
-        ds[v] = unpack_lo<T>(pw[hh][e]) * (dp[v] - dl4[v / 4][v % 4]);
-        ds[v + 1] = unpack_hi<T>(pw[hh][e]) * (dp[v + 1] - dl4[(v + 1) / 4][(v + 1) % 4]);
+        ds[v] = unpack_lo<T>(pw[hh][e]) * dp[v];
+        ds[v + 1] = unpack_hi<T>(pw[hh][e]) * dp[v + 1];
       }
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh)
@@ -765,8 +765,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
         block_flags(t, mbk, on, masked);
         u32x4 dsf[2], tf[2 * DB];
         f32x16 dp;
-        f32x4 dl4[4];
-        if (on) ds_first(base, mbk, dp, tf, dl4);
+        if (on) ds_first(base, mbk, dp, tf);
         if (mbk == 1) dma_wait();
         lds_barrier();
         if (mbk == 0 && t + 1 < ntiles) {
@@ -774,7 +773,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
           load_part(t + 1, 3);
         }
         if (on) {
-          ds_second(mbk, dp, dl4, dsf);
+          ds_second(mbk, dp, dsf);
           accumulate(tf, dsf);
         }
       }
