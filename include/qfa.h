@@ -56,6 +56,8 @@ const char *qfa_last_error(void);
  *   rowsum    nullable; [B*H*N] int32 sum of the token's codes (feeds the zero-point
  *             cross term of qfa_attn_fwd / qfa_attn_bwd; not produced by the reference)
  *   D in {32, 64, 128, 256}.  x and codes 16-byte aligned, strides multiples of 16 bytes.
+ * A token row that holds an infinity or a NaN gets unspecified codes (the formulas above send NaN through
+ * roundf and the int8 conversion, in the reference as here); the other rows are not affected.
  */
 int qfa_quant_per_token(const void *x, int x_dtype, int8_t *codes, float *scale_f32, void *scale_lp,
                         int scale_lp_dtype, int8_t *zp, int32_t *rowsum, int64_t B, int64_t H, int64_t N,
