@@ -182,7 +182,7 @@ int qfa_bwd_delta(const void *o, const void *dout, float *delta, int io_dtype, i
  * kernel, :207-237 wrapper); the reference's single dKV tensor is dK + dV (:161).
  *   workspace  caller-owned scratch of at least qfa_attn_bwd_workspace_bytes(B,H,Nq,Nk,D) bytes,
  *              16-byte aligned, overwritten: two staging passes fill it with delta = rowsum(O o dO),
- *              the transposed 16-bit tiles dO^T, Q^^T, K^^T (the dequantized Q and K rounded to
+ *              the transposed 16-bit tiles Q^^T, K^^T (the dequantized Q and K rounded to
  *              io_dtype, the operands of the dK and dQ products) and per-token constants, once
  *              per call, so that the two MFMA kernels stream ready-made tiles.  The scores S, and
  *              with them P, come from the INT8 codes exactly as in the forward.

@@ -1,8 +1,8 @@
 // Backward kernels for gfx950: two staging passes, then two MFMA kernels that recompute
 // P = exp(S - LSE) from the INT8 codes exactly as the forward does.
 //
-//   prep_q       per 64-query tile: delta = rowsum(O o dO) in fp32; dO^T and Qz^T = ((Qc - zq) * sq)^T as
-//                16-bit tiles [d][query] in the key order the MFMA layouts want; per-query constants
+//   prep_q       per 64-query tile: delta = rowsum(O o dO) in fp32; Qz^T = ((Qc - zq) * sq)^T as a
+//                16-bit tile [d][query] in the key order the MFMA layouts want; per-query constants
 //   prep_k       per 64-key tile: Kz^T = ((Kc - zk) * sk)^T likewise; per-key constants
 //                (both write into the caller's workspace; every tile is converted and transposed
 //                once instead of once per consuming workgroup)
@@ -10,12 +10,13 @@
 //                S^T = Kc.Qc^T (INT8 MFMA), dP^T = V.dO^T, dS^T = P^T o (dP^T - delta),
 //                dQ^T += Kz^T.dS^T                with Kz = (Kc - zk) * sk, the dequantized K rounded to 16 bits
 //   dkdv kernel  one workgroup = 128 keys (32 per wave), loops over 64-query tiles.
-//                S = Qc.Kc^T (INT8 MFMA), dP = dO.V^T, dV^T += dO^T.P,
+//                S = Qc.Kc^T (INT8 MFMA), dP = dO.V^T, dV^T += dO^T.P (dO^T read out of the dO tile by
+//                the transposing LDS reads),
 //                dK^T += Qz^T.dS                  with Qz = (Qc - zq) * sq, the dequantized Q rounded to 16 bits
 // In both, the wave's own operand (queries resp. keys) stays in registers as the MFMA B operand
 // for the whole loop and the streamed operand comes from LDS as the A operand.  The 32x32
 // accumulator layout then leaves P / dS in registers exactly in the B-operand layout of the next
-// product; the transposed LDS tiles (Kz^T, dO^T, Qz^T) are written in the matching permuted order.
+// product; the transposed LDS tiles (Kz^T, Qz^T) are written in the matching permuted order.
 // dQ is produced by its own kernel instead of atomics, so results are deterministic.
 // The scales of the streamed operand are folded into its transposed 16-bit tile (Kz^T, Qz^T) by the staging
 // pass, so dS is used as it comes: the tiles then hold the dequantized K and Q rounded to the 16-bit type, the
@@ -90,7 +91,7 @@ template <int D> struct BwdWs {
   static constexpr int T_BYTES = D * BWD_TILE * 2;            // one transposed tile
   static constexpr int CQ_BYTES = 5 * BWD_TILE * 4;           // digits (2 dwords/query), a, -lse*log2e, -delta
   static constexpr int CK_BYTES = 3 * BWD_TILE * 4;           // digits (2 dwords/key), key scale
-  static constexpr int Q_BLOB = 2 * T_BYTES + CQ_BYTES;       // dO^T, Qz^T, constants
+  static constexpr int Q_BLOB = T_BYTES + CQ_BYTES;           // Qz^T, constants
   static constexpr int K_BLOB = T_BYTES + CK_BYTES;           // Kz^T, constants
 };
 
@@ -140,22 +141,6 @@ __device__ __forceinline__ void store_codes_transposed(const u32x2 (&c)[4], cons
     *reinterpret_cast<u32x2 *>(dst + e * stride) = o;
   }
 }
-// 4 rows x 8 columns of 16-bit floats (one 16-byte register per row), transposed the same way
-__device__ __forceinline__ void store_16b_transposed(const u32x4 (&w)[4], unsigned char *dst, int stride) {
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const int x = e / 2;
-    u32x2 o;
-    if (e % 2 == 0) {
-      o[0] = (w[0][x] & 0xffffu) | (w[1][x] << 16);
-      o[1] = (w[2][x] & 0xffffu) | (w[3][x] << 16);
-    } else {
-      o[0] = (w[0][x] >> 16) | (w[1][x] & 0xffff0000u);
-      o[1] = (w[2][x] >> 16) | (w[3][x] & 0xffff0000u);
-    }
-    *reinterpret_cast<u32x2 *>(dst + e * stride) = o;
-  }
-}
 // integer n -> (128*floor(n/128), n mod 128) resp. their negatives, as a packed pair of 16-bit floats
 template <typename T> __device__ __forceinline__ unsigned base128_pair(int n, float sign) {
   const int hi = n >> 7, lo = n & 127;
@@ -163,7 +148,7 @@ template <typename T> __device__ __forceinline__ unsigned base128_pair(int n, fl
 }
 
 // ------------------------------------------------------------------------------------------ prep
-// One block per (b,h, 64-query tile): delta, dO^T, Qz^T and the per-query constants.
+// One block per (b,h, 64-query tile): delta, Qz^T and the per-query constants.
 template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_q_kernel(BwdArgs a) {
   typedef BwdWs<D> WS;
   __shared__ float red[D / 8][BWD_TILE];
@@ -198,9 +183,8 @@ template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_q_k
       red[dc][4 * r4 + r] = s;
     }
     const int pos = perm_pos4(r4);
-    store_16b_transposed(greg, blob + (dc * 8) * (BWD_TILE * 2) + pos * 2, BWD_TILE * 2);
     // the dequantized Q itself, rounded to the 16-bit type (what dK = sm * dS^T Q^ contracts with)
-    store_codes_transposed<T>(creg, zreg, sreg, blob + WS::T_BYTES + (dc * 8) * (BWD_TILE * 2) + pos * 2, BWD_TILE * 2);
+    store_codes_transposed<T>(creg, zreg, sreg, blob + (dc * 8) * (BWD_TILE * 2) + pos * 2, BWD_TILE * 2);
   }
   __syncthreads();
   if (tid < BWD_TILE) {
@@ -210,7 +194,7 @@ template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_q_k
     for (int x = 0; x < D / 8; ++x) delta += red[x][tid];
     const int zq = (int)a.zq[tq0 + i];
     const int c = a.rq[tq0 + i] - D * zq;
-    unsigned *cq = reinterpret_cast<unsigned *>(blob + 2 * WS::T_BYTES);
+    unsigned *cq = reinterpret_cast<unsigned *>(blob + WS::T_BYTES);
     u32x2 dg;
     dg[0] = pack2<T>((float)(-zq), (float)(-zq));      // k-group 0: times the two digits of rk
     dg[1] = base128_pair<T>(c, -1.0f);                 // k-group 1: minus the digits of rq - D*zq, times zk
@@ -320,7 +304,7 @@ __global__ __launch_bounds__(DqShape<D>::THREADS, DqShape<D>::WAVES_PER_SIMD) vo
   for (int kd = 0; kd < KD; ++kd)
     dof[kd] = *reinterpret_cast<const u32x4 *>(do_bh + (int64_t)qi_c * a.sdon + kd * 16 + g * 8);
   // per-query constants prepared by prep_q: correction digits, a = sq*sm*log2e, -lse*log2e, -delta
-  const unsigned *cq = reinterpret_cast<const unsigned *>(wsq_bh + (int64_t)(qi_c / BWD_TILE) * WS::Q_BLOB + 2 * WS::T_BYTES);
+  const unsigned *cq = reinterpret_cast<const unsigned *>(wsq_bh + (int64_t)(qi_c / BWD_TILE) * WS::Q_BLOB + WS::T_BYTES);
   const int ql = qi_c % BWD_TILE;
   const u32x4 corr_q = {cq[2 * ql + g], 0u, 0u, 0u};
   const float a_i = __builtin_bit_cast(float, cq[2 * BWD_TILE + ql]);
@@ -501,11 +485,11 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
   constexpr int NP = DkvShape<D>::PAIRS, DKV_THREADS = DkvShape<D>::THREADS;
   typedef BwdWs<D> WS;
   typedef Swz<D> SQ;            // Q code rows
-  typedef Swz<2 * D> SG;        // dO rows
+  typedef SwzDual<2 * D> SG;    // dO rows: read row-wise for dP and through transposing reads for dV
   typedef Swz<BWD_TILE * 2> ST; // transposed rows
   constexpr int KS = D / 32, DB = D / 32, KD = D / 16;
   constexpr int Q_BYTES = BWD_TILE * D, G_BYTES = BWD_TILE * 2 * D, T_BYTES = WS::T_BYTES;
-  constexpr int OFF_DO = Q_BYTES, OFF_DOT = OFF_DO + G_BYTES, OFF_QT = OFF_DOT + T_BYTES, OFF_C = OFF_QT + T_BYTES,
+  constexpr int OFF_DO = Q_BYTES, OFF_QT = OFF_DO + G_BYTES, OFF_C = OFF_QT + T_BYTES,
                 BUF = OFF_C + WS::CQ_BYTES;
   constexpr int OFF_X = 2 * BUF;             // P exchange: per pair 2 slots x 64 lanes x 16 packed 16-bit floats
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF + NP * 4096];
@@ -566,14 +550,14 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
   // full tiles: per-thread offsets computed once, one copy instruction per chunk afterwards
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   TileCopy<D, BWD_TILE, DKV_THREADS> cp_q;
-  TileCopy<2 * D, BWD_TILE, DKV_THREADS> cp_g;
+  TileCopy<2 * D, BWD_TILE, DKV_THREADS, SG> cp_g;
   TileCopy<BWD_TILE * 2, D, DKV_THREADS> cp_t;
   TileCopy<WS::CQ_BYTES, 1, DKV_THREADS, NoSwz<WS::CQ_BYTES>> cp_c;
   cp_q.init((unsigned)a.sqn, tid);
   cp_g.init((unsigned)a.sdon * 2u, tid);
   cp_t.init(BWD_TILE * 2, tid);
   cp_c.init(0, tid);
-  // the copy of a tile goes out in two halves (parts 0-1, 2-3), one before each 32-query block of the
+  // the copy of a tile goes out in two halves (parts 0-1, 2), one before each 32-query block of the
   // tile in work, so that the memory pipe is not handed all of it in one burst (four quarters, one
   // per phase, measured slower)
   auto load_part = [&](int t, int part) {
@@ -583,18 +567,16 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
     if (part == 0) {
       if (full) cp_q.issue(qc_bh + (int64_t)t * BWD_TILE * a.sqn, base, wave_u, tid);
       else dma_rows<D, BWD_TILE, DKV_THREADS>(qc_bh, a.sqn, t * BWD_TILE, a.Nq - 1, base, tid);
-      cp_c.issue(blob + 2 * WS::T_BYTES, base + OFF_C, wave_u, tid);
+      cp_c.issue(blob + WS::T_BYTES, base + OFF_C, wave_u, tid);
     } else if (part == 1) {
       if (full) cp_g.issue(do_bh + (int64_t)t * BWD_TILE * a.sdon * 2, base + OFF_DO, wave_u, tid);
-      else dma_rows<2 * D, BWD_TILE, DKV_THREADS>(do_bh, a.sdon * 2, t * BWD_TILE, a.Nq - 1, base + OFF_DO, tid);
+      else dma_rows<2 * D, BWD_TILE, DKV_THREADS, SG>(do_bh, a.sdon * 2, t * BWD_TILE, a.Nq - 1, base + OFF_DO, tid);
     } else if (part == 2) {
-      cp_t.issue(blob, base + OFF_DOT, wave_u, tid);
-    } else {
-      cp_t.issue(blob + WS::T_BYTES, base + OFF_QT, wave_u, tid);
+      cp_t.issue(blob, base + OFF_QT, wave_u, tid);
     }
   };
   auto load_tile = [&](int t) {
-    for (int part = 0; part < 4; ++part) load_part(t, part);
+    for (int part = 0; part < 3; ++part) load_part(t, part);
   };
 
   f32x16 oacc[DB];   // dV^T (P role) or dK^T (dS role) for this lane's key
@@ -610,9 +592,16 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
   // LDS operands are fetched in groups well ahead of the MFMAs that consume them (a 16-byte LDS read
   // takes far longer than an MFMA issue slot, and the compiler keeps loads next to their use), the
   // groups are pinned in place with scheduling barriers.
-  // ---- P role, first half of a block: S, correction, P; P goes to LDS (fp32) and stays packed in pf;
-  // the dO^T fragments of the second half are fetched here as well
-  auto p_first = [&](const unsigned char *base, int i0, int mbk, u32x4 (&pf)[2], u32x4 (&tf)[2 * DB], auto masked_tag) {
+  // ---- P role, first half of a block: S, correction, P; P goes to LDS and stays packed in pf;
+  // the dO^T fragments of the second half are requested here as well
+  // dO^T comes out of the dO tile through ds_read_b64_tr_b16: lane (d, k-group g) gets queries
+  // 16hh + 4g + {0..3} and those + 8 of its d, the order in which pf holds P.  Offsets inside the tile:
+  const int t_row = (lane % 16) / 4;
+  const unsigned t_off = (unsigned)((4 * g + t_row) * (2 * D) +
+                                    ((((SG::quarter(t_row)) << 2) | ((2 * ((lane / 16) % 2) + (lane % 4) / 2) ^ g)) << 4) +
+                                    8 * (lane % 2));   // XOR 64*db: d block; XOR 32 with +8 rows: the second four queries
+  auto p_first = [&](const unsigned char *base, int i0, int mbk, u32x4 (&pf)[2], u32x2 (&ta)[2 * DB], u32x2 (&tb)[2 * DB],
+                     auto masked_tag) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     const unsigned *dgp = reinterpret_cast<const unsigned *>(base + OFF_C);
     const float *cs = reinterpret_cast<const float *>(base + OFF_C);
@@ -659,11 +648,17 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
       xch0[mbk * 128 + hh * 64 + lane] = pf[hh];
     }
     __builtin_amdgcn_sched_barrier(0);
+    // requested behind the compiler's back; the barrier that follows waits for every LDS operation of the
+    // wave, and lds_wait_async after it ties the registers to that wait
+    const unsigned tbase = lds_addr(base + OFF_DO) + mbk * 32 * (2 * D);
 #pragma unroll
-    for (int hh = 0; hh < 2; ++hh)
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-        tf[hh * DB + db] = *reinterpret_cast<const u32x4 *>(base + OFF_DOT + ST::off(32 * db + lr, 4 * mbk + 2 * hh + g));
+    for (int db = 0; db < DB; ++db) {
+      const unsigned ad = tbase + (t_off ^ (64 * db)), ad2 = tbase + (t_off ^ (64 * db) ^ 32);
+      ta[2 * db] = lds_read_tr16_async<0>(ad);
+      ta[2 * db + 1] = lds_read_tr16_async<8 * 2 * D>(ad2);
+      tb[2 * db] = lds_read_tr16_async<16 * 2 * D>(ad);
+      tb[2 * db + 1] = lds_read_tr16_async<24 * 2 * D>(ad2);
+    }
   };
   // ---- dS role, first half: dP = dO.V^T; then the Qz^T fragments and constants of the second half
   auto ds_first = [&](const unsigned char *base, int mbk, f32x16 &dp, u32x4 (&tf)[2 * DB]) {
@@ -738,18 +733,27 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
         }
         bool on, masked;
         block_flags(t, mbk, on, masked);
-        u32x4 pf[2], tf[2 * DB];
+        u32x4 pf[2];
+        u32x2 ta[2 * DB], tb[2 * DB];
         if (on) {
-          if (masked) p_first(base, t * BWD_TILE, mbk, pf, tf, std::true_type{});
-          else p_first(base, t * BWD_TILE, mbk, pf, tf, std::false_type{});
+          if (masked) p_first(base, t * BWD_TILE, mbk, pf, ta, tb, std::true_type{});
+          else p_first(base, t * BWD_TILE, mbk, pf, ta, tb, std::false_type{});
         }
         if (mbk == 1) dma_wait();
         lds_barrier();   // P of this block is in LDS
         if (mbk == 0 && t + 1 < ntiles) {
           load_part(t + 1, 2);
-          load_part(t + 1, 3);
         }
-        if (on) accumulate(tf, pf);
+        if (on) {
+          lds_wait_async<0>(ta);
+          lds_wait_async<0>(tb);
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+            oacc[db] = mfma_16b<T>(u32x4{ta[2 * db][0], ta[2 * db][1], ta[2 * db + 1][0], ta[2 * db + 1][1]}, pf[0], oacc[db]);
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+            oacc[db] = mfma_16b<T>(u32x4{tb[2 * db][0], tb[2 * db][1], tb[2 * db + 1][0], tb[2 * db + 1][1]}, pf[1], oacc[db]);
+        }
       }
     }
   } else {
@@ -770,7 +774,6 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
         lds_barrier();
         if (mbk == 0 && t + 1 < ntiles) {
           load_part(t + 1, 2);
-          load_part(t + 1, 3);
         }
         if (on) {
           ds_second(mbk, dp, dsf);
@@ -824,9 +827,9 @@ template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStre
   {
     constexpr int DKV_THREADS = DkvShape<D>::THREADS;
     a.nblocks = (int)((x.Nk + DkvShape<D>::BLK - 1) / DkvShape<D>::BLK);
-    // per head the kernel streams Qc, dO, dO^T and Qz^T (7 bytes per query and d): group heads while that
+    // per head the kernel streams Qc, dO and Qz^T (5 bytes per query and d): group heads while that
     // stays within an XCD's 4 MB L2 (one head already fills it at N=4096, D=128)
-    const int64_t head_bytes = x.Nq * (int64_t)D * 7;
+    const int64_t head_bytes = x.Nq * (int64_t)D * 5;
     a.group_log2 = 0;
     while (a.group_log2 < 2 && (head_bytes << (a.group_log2 + 1)) <= (4 << 20)) ++a.group_log2;
     const int64_t total = (int64_t)a.nblocks * BH;

@@ -136,6 +136,19 @@ template <int ROW_BYTES> struct SwzQuad {
   static __device__ __forceinline__ int swz(int row) { return 4 * ((row / RPL) % QPR); }
 };
 
+// Layout for a [row][d] tile of 16-bit floats that is read BOTH ways: row-wise (16 lanes = 16 consecutive
+// rows at one logical chunk) and through the transposing reads (32 lanes = 4 consecutive rows x 64
+// contiguous bytes).  The row's low bits move the 64-byte quarter, bits 2-3 the chunk inside the quarter, so
+// either pattern lands on 16 different 16-byte slots of the 256-byte bank line.
+template <int ROW_BYTES> struct SwzDual {
+  static_assert(ROW_BYTES == 256 || ROW_BYTES == 128, "rows of 128 or 64 16-bit floats");
+  static constexpr int CPR = ROW_BYTES / 16;
+  // the part of the XOR that moves quarters (a function of the row's low bits only)
+  static __device__ __forceinline__ int quarter(int row) { return ROW_BYTES == 256 ? (row & 3) : ((row >> 1) & 1); }
+  static __device__ __forceinline__ int swz(int row) { return (quarter(row) << 2) | ((row >> 2) & 3); }
+  static __device__ __forceinline__ int off(int r, int c) { return r * ROW_BYTES + ((c ^ swz(r)) << 4); }
+};
+
 // rows [row0, row0+ROWS) (clamped to row_max) of a row-major global array -> swizzled LDS tile; NT threads
 template <int ROW_BYTES, int ROWS, int NT, typename S = Swz<ROW_BYTES>>
 __device__ __forceinline__ void dma_rows(const unsigned char *g, int64_t gstride, int row0, int row_max,
