@@ -13,7 +13,8 @@
  *   - Return value: 0 = success, < 0 = one of the QFA_E* argument errors (nothing was
  *     launched), > 0 = the hipError_t of a failed launch.  qfa_last_error() returns a
  *     thread-local, human readable description of the last failure on this thread.
- *   - The library keeps no mutable global state; calls from several host threads are safe.
+ *   - The library keeps no mutable global state and calls from several host threads are safe; the one
+ *     exception is qfa_attn_fwd_shared_kv_static, which owns a static device scratch array (see there).
  *
  * Reference interface each entry point replaces (paths in yisunlp/quant_flash_attn):
  * the reference has no FFI; the boundary is the Triton launch made by its Python operators.
@@ -124,6 +125,25 @@ int qfa_attn_fwd_shared_kv(const void *q, const int8_t *codes, const void *scale
                            int64_t sqb, int64_t sqh, int64_t sqn, int64_t scb, int64_t sch, int64_t scn, int64_t sob,
                            int64_t soh, int64_t son, float sm_scale, void *workspace, int64_t workspace_bytes,
                            void *stream);
+
+/*
+ * qfa_attn_fwd_shared_kv for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): no counterpart in the reference.  Same
+ * computation, same kernels and bit-identical results as qfa_attn_fwd_shared_kv given a workspace, but the
+ * partial results of a split over keys live in a static device array of QFA_STATIC_SCRATCH_BYTES inside the
+ * library (every GPU the library runs on holds its own copy until the process ends).  The call allocates
+ * and frees nothing; its first use on a device looks up that array's device address (hipGetSymbolAddress)
+ * and keeps it.  A shape whose split needs more than QFA_STATIC_SCRATCH_BYTES
+ * (qfa_attn_fwd_shared_kv_workspace_bytes tells) is rejected with QFA_EUNSUPPORTED before anything is
+ * launched.  All calls on one GPU share the one array: calls that overlap in time on the same GPU (two
+ * streams, two threads) race on it -- serialise them, or use the workspace form.  Nothing in the array has
+ * to be cleared between calls (every partial result is written before it is read).
+ */
+#define QFA_STATIC_SCRATCH_BYTES (16 << 20)
+int qfa_attn_fwd_shared_kv_static(const void *q, const int8_t *codes, const void *scale, int scale_dtype,
+                                  const int8_t *zp, void *o, float *lse, int io_dtype, int64_t B, int64_t H, int64_t Nq,
+                                  int64_t Nk, int D, int64_t sqb, int64_t sqh, int64_t sqn, int64_t scb, int64_t sch,
+                                  int64_t scn, int64_t sob, int64_t soh, int64_t son, float sm_scale, void *stream);
 
 /*
  * Backward of qfa_attn_fwd_shared_kv, fp16:

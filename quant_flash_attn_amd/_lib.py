@@ -29,6 +29,7 @@ _SIGNATURES = {
     "qfa_attn_fwd": (c_int, [_P] * 11 + [_I, _L, _L, _L, _L, _I] + [_L] * 12 + [_F, _I, _P]),
     "qfa_attn_fwd_shared_kv_workspace_bytes": (c_int64, [_L, _L, _L, _L, _I]),
     "qfa_attn_fwd_shared_kv": (c_int, [_P, _P, _P, _I, _P, _P, _P, _I, _L, _L, _L, _L, _I] + [_L] * 9 + [_F, _P, _L, _P]),
+    "qfa_attn_fwd_shared_kv_static": (c_int, [_P, _P, _P, _I, _P, _P, _P, _I, _L, _L, _L, _L, _I] + [_L] * 9 + [_F, _P]),
     "qfa_attn_bwd_shared_kv": (c_int, [_P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _P, _L, _L, _L, _L, _I] + [_L] * 18
                                + [_F, _P]),
     "qfa_bench_qk_stage": (c_int, [_P] * 11 + [_I, _L, _L, _L, _L, _I] + [_L] * 12 + [_F, _I, _P]),

@@ -168,6 +168,20 @@ int qfa_attn_fwd_shared_kv(const void *q, const int8_t *codes, const void *scale
   return launch_skv_fwd(a, (hipStream_t)stream);
 }
 
+int qfa_attn_fwd_shared_kv_static(const void *q, const int8_t *codes, const void *scale, int scale_dtype,
+                                  const int8_t *zp, void *o, float *lse, int io_dtype, int64_t B, int64_t H, int64_t Nq,
+                                  int64_t Nk, int D, int64_t sqb, int64_t sqh, int64_t sqn, int64_t scb, int64_t sch,
+                                  int64_t scn, int64_t sob, int64_t soh, int64_t son, float sm_scale, void *stream) {
+  SkvAttnArgs a;
+  memset(&a, 0, sizeof(a));
+  a.q = q; a.codes = codes; a.scale = scale; a.zp = zp; a.o = o; a.lse = lse;
+  a.B = B; a.H = H; a.Nq = Nq; a.Nk = Nk; a.D = D; a.io_dtype = io_dtype; a.scale_dtype = scale_dtype;
+  a.sqb = sqb; a.sqh = sqh; a.sqn = sqn; a.scb = scb; a.sch = sch; a.scn = scn; a.sob = sob; a.soh = soh; a.son = son;
+  a.sm_scale = sm_scale;
+  if (int e = check_shared_kv("attn_fwd_shared_kv_static", a)) return e;
+  return launch_skv_fwd_static(a, (hipStream_t)stream);
+}
+
 int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp,
                            const void *o, const void *dout, const float *lse, void *dq, void *dkv, int io_dtype,
                            int grad_dtype, const float *grad_scale,

@@ -56,6 +56,8 @@ struct SkvAttnArgs {
 };
 int launch_skv_fwd(const SkvAttnArgs &a, hipStream_t st);
 int64_t skv_fwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D);
+// the same with the partial results of a split in the library's own static device array (a.workspace is ignored)
+int launch_skv_fwd_static(const SkvAttnArgs &a, hipStream_t st);
 int launch_skv_bwd(const SkvAttnArgs &a, hipStream_t st);        // io_dtype QFA_F16, Nq <= 32: one fused pass
 int launch_skv_bwd_long(const SkvAttnArgs &a, hipStream_t st);   // io_dtype QFA_F16, any Nq: dQ kernel + dKV kernel
 

@@ -24,6 +24,7 @@
 //
 // V^T fragments come out of the row-major code tile through ds_read_b64_tr_b8: inside a group of 16
 // lanes, lane i receives byte i%8 of the 8-byte rows addressed by lanes (i%16)/8 + {0,2,..,14}.
+#include <mutex>
 #include <type_traits>
 
 #include "qfa_host.h"
@@ -416,6 +417,52 @@ template <typename T, typename S, int D> static int launch_skv_fwd_tsd(const Skv
 template <typename T, int D> static int launch_skv_fwd_td(const SkvAttnArgs &x, hipStream_t st) {
   if (x.scale_dtype == QFA_F32) return launch_skv_fwd_tsd<T, float, D>(x, st);
   return launch_skv_fwd_tsd<T, T, D>(x, st);   // validated: scale_dtype == io_dtype
+}
+
+// ---- scratch for callers that cannot allocate --------------------------------------------------------
+// The split over keys needs device memory beyond the inputs and outputs (the partial results).  This array
+// is that memory for qfa_attn_fwd_shared_kv_static: every GPU the library runs on holds its own copy until
+// the process ends.  In host code the array's NAME is only a stand-in for the symbol; the device address is
+// asked for once per device (with that device current) and only that address is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[QFA_STATIC_SCRATCH_BYTES];
+
+static constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void *g_scratch_ptr[kMaxDevices];   // device address of `scratch` on device i, nullptr until asked for
+
+// Device address of the current device's scratch array (0 and the address in *out, or an error code).
+static int static_scratch(void **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return set_error((int)e, "attn_fwd_shared_kv_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return set_error(QFA_EUNSUPPORTED, "attn_fwd_shared_kv_static: device index %d outside [0, %d)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return set_error(e != hipSuccess ? (int)e : QFA_EINVAL, "attn_fwd_shared_kv_static: hipGetSymbolAddress: %s",
+                       hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+int launch_skv_fwd_static(const SkvAttnArgs &x, hipStream_t st) {
+  const int64_t need = skv_fwd_workspace_bytes(x.B, x.H, x.Nq, x.Nk, x.D);
+  if (need > (int64_t)QFA_STATIC_SCRATCH_BYTES)
+    return set_error(QFA_EUNSUPPORTED,
+                     "attn_fwd_shared_kv_static: this shape splits its keys into partial results of %lld bytes, more "
+                     "than the built-in scratch of %lld bytes; use qfa_attn_fwd_shared_kv with a caller workspace",
+                     (long long)need, (long long)QFA_STATIC_SCRATCH_BYTES);
+  SkvAttnArgs y = x;
+  y.workspace = nullptr;
+  if (need > 0) {   // every partial result is written by the first kernel before the merge reads it: nothing to clear
+    if (int e = static_scratch(&y.workspace)) return e;
+  }
+  return launch_skv_fwd(y, st);
 }
 
 int launch_skv_fwd(const SkvAttnArgs &x, hipStream_t st) {
