@@ -86,7 +86,8 @@ int qfa_dequant_per_token(const int8_t *codes, const void *scale, int scale_dtyp
  *   qc,kc  int8 [B,H,Nq|Nk,D];  sq,sk float, zq,zk int8, rq,rk int32: dense [B*H*Nq|Nk]
  *   v, o   [B,H,Nk|Nq,D] of io_dtype (QFA_BF16 or QFA_F16);  lse float [B*H*Nq]
  *   D in {64, 128}.  causal != 0 requires Nq == Nk.  All tensors 16-byte aligned, strides
- *   multiples of 16 bytes, token strides below 2^23 elements (QFA_EUNSUPPORTED otherwise).
+ *   multiples of 16 bytes, token strides below 2^23 elements, Nq and Nk at most 2^28
+ *   (QFA_EUNSUPPORTED otherwise).
  */
 int qfa_attn_fwd(const int8_t *qc, const float *sq, const int8_t *zq, const int32_t *rq, const int8_t *kc,
                  const float *sk, const int8_t *zk, const int32_t *rk, const void *v, void *o, float *lse,
@@ -112,6 +113,9 @@ int qfa_attn_fwd(const int8_t *qc, const float *sq, const int8_t *zq, const int3
  *   The codes' binary16 offset (1152) is removed through the sum of a query's D elements: |sum| must
  *   stay below 2^21, and the scores carry an absolute error of a few fp32 ulp of 1152 * |sum| code
  *   units (nothing for |q| of order 10; about a percent of a score once every element is near 500).
+ *   Binary16 ranges, not checked: the queries enter the products as binary16 (a bf16 query above 65504 in
+ *   magnitude becomes an infinity and the row NaN), and the probabilities are multiplied by the key scale
+ *   before they are packed to binary16 (p * scale below 65504: scales up to about 4e3).  Nq, Nk at most 2^28.
  *   workspace  nullable.  With few (batch, head) pairs one workgroup per 16 queries leaves most of the
  *              chip idle (the reference launches one program per (batch, head)); given a caller-owned
  *              scratch of qfa_attn_fwd_shared_kv_workspace_bytes(...) bytes (16-byte aligned; the
@@ -162,6 +166,12 @@ int qfa_attn_fwd_shared_kv_static(const void *q, const int8_t *codes, const void
  *               over dO * 2^k and *grad_scale = 2^-k without a host synchronisation;
  *   codes, scale, scale_dtype, zp, lse as in the forward.  D in {64, 128, 256} (256: one pass up to 16 queries).
  *   The sums of a query's and of a dO row's D elements must stay inside binary16 range.
+ *   Range of dout: the kernels do not multiply by dO itself but by  ds = sm_scale * p * (dP - delta)  and by
+ *   ds * scale_j,  both packed to binary16 (the reference rounds ds to fp16 as well, quant_flash_attn.py:159).
+ *   With |dO| well below one these operands fall into binary16's subnormals and the gradients lose precision
+ *   (a few percent at |dO| ~ 2^-6 for unit-variance K = V, everything at 2^-14).  dQ and dKV are linear in dO:
+ *   hand over dO * 2^k with the largest |dO| * 2^k * max(scale) near 8 (and |dO| * 2^k below 2^14) and
+ *   *grad_scale = 2^-k, as the Python entry point does on the device.
  */
 int qfa_attn_bwd_shared_kv(const void *q, const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp,
                            const void *o, const void *dout, const float *lse, void *dq, void *dkv, int io_dtype,

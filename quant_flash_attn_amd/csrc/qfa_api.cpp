@@ -25,6 +25,7 @@ int check_launch(const char *what) {
   return (int)e;
 }
 
+static constexpr int64_t kMaxTokens = 1LL << 28;   // longest sequence (Nq, Nk) the attention entry points take
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static bool is_float_dtype(int d) { return d == QFA_F32 || d == QFA_F16 || d == QFA_BF16; }
 static int elem_size(int d) { return d == QFA_F32 ? 4 : 2; }
@@ -87,7 +88,9 @@ static int check_attn_common(const char *who, const AttnArgs &a) {
   if (a.io_dtype != QFA_BF16 && a.io_dtype != QFA_F16)
     return set_error(QFA_EINVAL, "%s: io_dtype must be QFA_BF16 or QFA_F16", who);
   if (a.B <= 0 || a.H <= 0 || a.Nq <= 0 || a.Nk <= 0) return set_error(QFA_EINVAL, "%s: B, H, Nq, Nk must be positive", who);
-  if (a.Nq > 0x7fffff00LL || a.Nk > 0x7fffff00LL) return set_error(QFA_EUNSUPPORTED, "%s: sequence too long", who);
+  // the kernels form byte offsets into the per-token vectors (4 bytes per token) in 31 bits
+  if (a.Nq > kMaxTokens || a.Nk > kMaxTokens)
+    return set_error(QFA_EUNSUPPORTED, "%s: sequences of more than 2^28 tokens are not supported", who);
   if (a.D != 64 && a.D != 128) return set_error(QFA_EUNSUPPORTED, "%s: head_dim %d not in {64, 128}", who, a.D);
   if (!(a.sm_scale > 0.0f) || !(a.sm_scale < 3.0e38f))
     return set_error(QFA_EINVAL, "%s: sm_scale must be a positive finite number", who);
@@ -127,7 +130,9 @@ static int check_shared_kv(const char *who, const SkvAttnArgs &a) {
   if (a.scale_dtype != QFA_F32 && a.scale_dtype != a.io_dtype)
     return set_error(QFA_EINVAL, "%s: scale_dtype must be QFA_F32 or equal to io_dtype", who);
   if (a.B <= 0 || a.H <= 0 || a.Nq <= 0 || a.Nk <= 0) return set_error(QFA_EINVAL, "%s: B, H, Nq, Nk must be positive", who);
-  if (a.Nq > 0x7fffff00LL || a.Nk > 0x7fffff00LL) return set_error(QFA_EUNSUPPORTED, "%s: sequence too long", who);
+  // the kernels form byte offsets into the per-token vectors (4 bytes per token) in 31 bits
+  if (a.Nq > kMaxTokens || a.Nk > kMaxTokens)
+    return set_error(QFA_EUNSUPPORTED, "%s: sequences of more than 2^28 tokens are not supported", who);
   if (a.D != 64 && a.D != 128 && a.D != 256)
     return set_error(QFA_EUNSUPPORTED, "%s: head_dim %d not in {64, 128, 256}", who, a.D);
   if (!(a.sm_scale > 0.0f) || !(a.sm_scale < 3.0e38f))

@@ -281,18 +281,15 @@ class QuantFlashAttention(torch.autograd.Function):
         t = ctx.saved_tensors
         if ctx.shared_kv:
             q, codes, scale, zp, o, lse = t
-            if q.dtype == torch.float16:
-                dq, dkv = attn_bwd_shared_kv(q, codes, scale, zp, o, grad_output, lse, ctx.sm_scale)
-                return dq, dkv.to(ctx.kv_dtype), None, None
-            # bf16: the backward kernels compute in binary16.  q and o convert exactly (more mantissa, values
-            # of order one); dO may lie below binary16's range, so it is handed over scaled by a power of two
-            # chosen on the device from its largest magnitude (no synchronisation), and the kernels scale dQ
-            # and dKV -- linear in dO -- back while they round them to bf16.
-            do32 = grad_output.to(torch.float32)
-            k = torch.floor(torch.log2(256.0 / do32.abs().amax().clamp_min(1e-30))).clamp_(-100.0, 100.0)
-            dq, dkv = attn_bwd_shared_kv(q.to(torch.float16), codes, scale, zp, o.to(torch.float16),
-                                         (do32 * torch.exp2(k)).to(torch.float16), lse, ctx.sm_scale,
-                                         grad_dtype=torch.bfloat16, grad_scale=torch.exp2(-k))
+            # The backward kernels compute in binary16, and what they feed the matrix pipe is not dO but
+            # sm_scale * p * (dP - delta) and that times the key's scale: with dO as it comes, ordinary small
+            # gradients land in binary16's subnormals (or flush to zero) there.  dQ and dKV are linear in dO,
+            # so dO is handed over scaled by a power of two chosen on the device (no synchronisation) from
+            # its largest magnitude and from the largest key scale, and the kernels scale dQ and dKV back
+            # while they round them.  q and o convert exactly from bf16 (more mantissa, values of order one).
+            do16, back = _normalised_dout(grad_output, scale)
+            dq, dkv = attn_bwd_shared_kv(q.to(torch.float16), codes, scale, zp, o.to(torch.float16), do16, lse,
+                                         ctx.sm_scale, grad_dtype=q.dtype, grad_scale=back)
             return dq.to(ctx.q_dtype), dkv.to(ctx.kv_dtype), None, None
         else:
             qq, kq = QuantizedTokens(*t[0:4]), QuantizedTokens(*t[4:8])
@@ -300,6 +297,20 @@ class QuantFlashAttention(torch.autograd.Function):
         dq, dk, dv = attn_bwd_quantized(qq, kq, v16, o, grad_output.to(v16.dtype), lse, False, ctx.sm_scale)
         dkv = dk.to(torch.float32).add_(dv).to(ctx.kv_dtype)      # :161 (dk already carries sm_scale)
         return dq.to(ctx.q_dtype), dkv, None, None
+
+
+def _normalised_dout(grad_output: torch.Tensor, kv_scale: torch.Tensor):
+    """(dO * 2^k as float16, 2^-k as a one-element float32 tensor) for the binary16 backward kernels.
+
+    k puts the largest |dO| at 2^8 when the key scales are of the usual size (2^-5 for values of order
+    one) and higher when they are smaller, since the smallest operand the kernels form carries the
+    key scale as a factor; dO * 2^k itself stays below 2^14.  Everything is computed on the device."""
+    do32 = grad_output.to(torch.float32)
+    amax = do32.abs().amax().clamp_min(1e-30)
+    smax = kv_scale.to(torch.float32).abs().amax().clamp(1e-30, 2.0 ** -5)
+    k = torch.minimum(torch.floor(torch.log2(8.0 / (amax * smax))), torch.floor(torch.log2(16384.0 / amax)))
+    k = k.clamp_(-100.0, 100.0)
+    return (do32 * torch.exp2(k)).to(torch.float16), torch.exp2(-k)
 
 
 def _legacy_operands(q, codes, scale, zp, io):

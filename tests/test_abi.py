@@ -58,6 +58,11 @@ def test_argument_errors_need_no_gpu(qfa):
     s0 = (128 * 64 * 2, 128 * 64, 64)
     rc = L.qfa_attn_fwd(*([ok_ptr] * 11), 2, 1, 2, 128, 128, 64, *s0, *sb, *s0, *s0, 0.125, 0, None)
     assert rc == -2 and b"token strides" in L.qfa_last_error()
+    # sequences beyond 2^28 tokens: byte offsets into the per-token vectors would not fit 31 bits
+    long_n = (1 << 28) + 64
+    sl = (long_n * 64, long_n * 64, 64)
+    rc = L.qfa_attn_fwd(*([ok_ptr] * 11), 2, 1, 1, 128, long_n, 64, *s0, *sl, *sl, *s0, 0.125, 0, None)
+    assert rc == -2 and b"2^28" in L.qfa_last_error()
     rc = L.qfa_bwd_delta(None, ok_ptr, ok_ptr, 2, 1, 1, 8, 64, 512, 512, 64, 512, 512, 64, None)
     assert rc == -1
     # shared-KV entry points

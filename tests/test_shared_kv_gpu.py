@@ -143,6 +143,33 @@ def test_shared_kv_entry_point_bf16(qfa, do_scale, D):
     assert_close("dKV", kvd.grad.cpu().double() / do_scale, dkv_ref / do_scale, scaled=True)
 
 
+@pytest.mark.parametrize("do_scale,kv_scale,Nq", [(2.0 ** -6, 1.0, 16), (2.0 ** -10, 1.0, 16), (2.0 ** -14, 1.0, 16),
+                                                  (1.0, 2.0 ** -6, 16), (2.0 ** -10, 1.0, 70), (1.0, 2.0 ** -6, 70)])
+def test_shared_kv_entry_point_fp16_small_gradients(qfa, do_scale, kv_scale, Nq):
+    """fp16 tensors with ordinary small gradients (and small K = V): the binary16 kernels do not multiply by dO
+    itself but by sm_scale * p * (dP - delta) and that times the key scale, which underflow long before dO
+    does; the entry point scales dO by a power of two around them.  One pass (16 queries) and the dQ + dKV
+    kernels (70 queries); gradients compared in units of dO's scale."""
+    B, H, Nk, D = 2, 3, 3000, 128
+    q, kv = _inputs("normal", B, H, Nq, Nk, D, torch.float16, seed=41)
+    kv = (kv.float() * kv_scale).to(torch.float16)
+    sm = 1.0 / math.sqrt(D)
+    qd = q.to(DEV).requires_grad_(True)
+    kvd = kv.to(DEV).requires_grad_(True)
+    kv_quant = qfa.asymmetric_quant_per_token(kvd.detach())
+    o = qfa.quant_flash_attn(qd, kvd, kv_quant, sm)
+    do = (torch.randn(o.shape, generator=torch.Generator().manual_seed(7)) * do_scale).to(torch.float16)
+    o.backward(do.to(DEV))
+    codes, scale, zp = (t.cpu() for t in kv_quant)
+    dq_ref, dkv_ref = oracle.legacy_bwd(q, codes, scale, zp, do, sm)
+    unit = do_scale * kv_scale            # dQ scales with dO and with K = V
+    # the gradients leave as float16 (as the reference's do): where they are tiny the reference values are
+    # rounded to that format first, subnormals and all, so that the comparison is about the kernels
+    r16 = lambda t: t.to(torch.float16).double()
+    assert_close("dQ", qd.grad.cpu().double() / unit, r16(dq_ref) / unit, scaled=True)
+    assert_close("dKV", kvd.grad.cpu().double() / do_scale, r16(dkv_ref) / do_scale, scaled=True)
+
+
 def test_shared_kv_entry_point_long_query_block(qfa):
     """97 queries (a reference test shape, test_accuracy.py:44): the forward splits them over workgroups
     of 16, the backward runs its dQ and dKV kernels."""
