@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the INT8 quantized flash-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all-configs] [--sdpa]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--quick]
 
 Workload (the configuration the headline metric is quoted on): B=4, H=32, N=4096, D=128, causal,
 bf16 q/k/v drawn N(0,1) plus a per-token mean offset N(0, 0.5), already resident in HBM.
@@ -17,7 +17,11 @@ The single JSON line printed last carries
                duration from HIP events recorded around every launch of the timed region
   cpu_baseline the reference's CPU-runnable path (torch eager quantize + dequantized SDPA,
                oracle.reference_cpu_path) timed on this machine's host cores on a bounded sample
-plus fwd+bwd, quantizer and kernel-only figures under "extra".
+plus, under "extra": backward and fwd+bwd figures, the quantizer, the QK^T stage alone, the other two GPU
+configurations (long context, small head dimension with its stand-alone quantizer rate), torch SDPA bf16 on the
+same GPU as the stated stand-in for the reference's Triton kernels (which cannot run these shapes), and the
+reference's own benchmark shape.  Before the warm-up steps the same step runs untimed for --settle-ms
+milliseconds (reported as settle_ms) so that a short run is not measured on a clock that is still ramping.
 """
 from __future__ import annotations
 
@@ -63,28 +67,51 @@ def time_events(fn, steps, warmup):
     return a.elapsed_time(b) / steps
 
 
-def cpu_baseline(cfg, budget_s=12.0):
-    """Reference CPU path on head-chunks of the same workload until ~budget_s of CPU time."""
-    from oracle import oracle
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(cfg, budget_s=10.0):
+    """Reference CPU path (torch eager quantize + dequantize + SDPA, oracle.reference_cpu_path) on head-chunks of
+    the same workload until ~budget_s of CPU time per leg: forward (the headline metric's step) and forward +
+    backward."""
+    from oracle import oracle   # the CPU baseline is the only leg of this file that touches the oracle
+    from quant_flash_attn_amd.synthetic import make_inputs
     B, H, N, D, causal = cfg["B"], cfg["H"], cfg["N"], cfg["D"], cfg["causal"]
     sm = 1.0 / math.sqrt(D)
     threads = torch.get_num_threads()
     chunk = 4
-    q, k, v, _ = oracle.make_inputs(cfg["dist"], 1, chunk, N, D, seed=1)
-    q, k, v = q.float(), k.float(), v.float()
-    with torch.no_grad():
-        oracle.reference_cpu_path(q[:, :1], k[:, :1], v[:, :1], causal, sm)      # warm-up
-        done, t0 = 0, time.perf_counter()
-        while True:
-            oracle.reference_cpu_path(q, k, v, causal, sm)
-            done += chunk
-            el = time.perf_counter() - t0
-            if el >= budget_s or done >= B * H:
-                break
+    q, k, v, do = (t.float() for t in make_inputs(cfg["dist"], 1, chunk, N, D, seed=1))
+
+    def leg(with_bwd):
+        run = (lambda a, b, c, d: oracle.reference_cpu_path(a, b, c, causal, sm, d)) if with_bwd else \
+              (lambda a, b, c, d: oracle.reference_cpu_path(a, b, c, causal, sm))
+        with torch.set_grad_enabled(with_bwd):
+            run(q[:, :1], k[:, :1], v[:, :1], do[:, :1])      # warm-up
+            done, t0 = 0, time.perf_counter()
+            while True:
+                run(q, k, v, do)
+                done += chunk
+                el = time.perf_counter() - t0
+                if el >= budget_s or done >= B * H:
+                    return done, el
+
+    done, el = leg(False)
+    done_b, el_b = leg(True)
     fl = flops_fwd(1, done, N, N, D, causal)
+    fl_b = 3.5 * flops_fwd(1, done_b, N, N, D, causal)
     return {"value": round(fl / el / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "cpu_model": cpu_model(),
             "sample": f"{done} of {B * H} (batch,head) slices of the same workload, N={N} D={D} "
-                      f"causal={causal}, fp32 torch eager quantize+dequantize+SDPA forward, {el:.1f} s"}
+                      f"causal={causal}, fp32 torch eager quantize+dequantize+SDPA forward, {el:.1f} s",
+            "fwd_bwd_value": round(fl_b / el_b / 1e12, 4),
+            "fwd_bwd_sample": f"{done_b} of {B * H} slices, the same plus .backward(dO), {el_b:.1f} s"}
 
 
 def main():
@@ -93,8 +120,12 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--all-configs", action="store_true", help="also time the long-context and D=64 configurations")
-    ap.add_argument("--sdpa", action="store_true", help="also time torch SDPA bf16 on the GPU (stand-in bar)")
+    ap.add_argument("--quick", action="store_true",
+                    help="skip the other configurations, the torch SDPA stand-in and the D=64 reference shape")
+    ap.add_argument("--settle-ms", type=float, default=300.0,
+                    help="untimed milliseconds of the same step before the warm-up steps (clock settling)")
+    ap.add_argument("--all-configs", action="store_true", help=argparse.SUPPRESS)   # now the default
+    ap.add_argument("--sdpa", action="store_true", help=argparse.SUPPRESS)          # now the default
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 256 MiB device-to-device copy (calibrates rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
@@ -107,14 +138,14 @@ def main():
         sys.exit(1)
 
     import quant_flash_attn_amd as qfa
-    from oracle import oracle   # only for synthetic inputs and the CPU-baseline leg
+    from quant_flash_attn_amd.synthetic import make_inputs
 
     dev = "cuda:0"
     torch.cuda.set_device(0)
     cfg = {"B": 4, "H": 32, "N": 4096, "D": 128, "causal": True, "dist": "offset"}
     B, H, N, D, causal = cfg["B"], cfg["H"], cfg["N"], cfg["D"], cfg["causal"]
     sm = 1.0 / math.sqrt(D)
-    q, k, v, do = (t.to(dev) for t in oracle.make_inputs(cfg["dist"], B, H, N, D, seed=0))
+    q, k, v, do = (t.to(dev) for t in make_inputs(cfg["dist"], B, H, N, D, seed=0))
     F_fwd = flops_fwd(B, H, N, N, D, causal)
     F_bwd = 2.5 * F_fwd                       # compute_flops.py:104
 
@@ -130,6 +161,13 @@ def main():
             evs[1].record()
         return qq, kq, o, lse
 
+    # untimed settling: the same step until settle_ms have passed, so that the clock the timed steps see is the
+    # one a long run sees (a 20-step run is 15 ms long; the shader clock takes longer than that to ramp)
+    settle_t0 = time.perf_counter()
+    while (time.perf_counter() - settle_t0) * 1e3 < args.settle_ms:
+        step()
+        torch.cuda.synchronize()
+    settle_ms = (time.perf_counter() - settle_t0) * 1e3
     for _ in range(args.warmup):
         step()
     events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
@@ -140,7 +178,8 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_step = (t1 - t0) * 1e3 / args.steps
-    ms_fwd_kernel = sum(a.elapsed_time(b) for a, b in events) / args.steps
+    launch_ms = sorted(a.elapsed_time(b) for a, b in events)
+    ms_fwd_kernel = sum(launch_ms) / args.steps
     value = F_fwd / (ms_step * 1e-3) / 1e12
 
     # ---- extras (outside the timed region)
@@ -199,10 +238,10 @@ def main():
                 "bwd_ms": round(mb, 4), "bwd_GBps": round(io_b / mb / 1e6, 1),
                 "bwd_frac_hbm_peak": round(io_b / mb / 1e6 / PEAK_HBM_GBS, 4), "bwd_tflops": round(2.5 * fl / mb / 1e9, 2)}
     extra["shared_kv_Z512_H16_Nq16_Nkv3000_D128_fp16"] = shared_kv_leg(128)
-    if args.all_configs:
+    if not args.quick:
         extra["shared_kv_Z512_H16_Nq16_Nkv3000_D64_fp16"] = shared_kv_leg(64)
 
-    if args.sdpa:
+    if not args.quick:
         import torch.nn.functional as Fn
         qs, ks, vs = (t.clone().requires_grad_(True) for t in (q, k, v))
         ms_s = time_events(lambda: Fn.scaled_dot_product_attention(qs.detach(), ks.detach(), vs.detach(), is_causal=causal, scale=sm), 20, 5)
@@ -217,12 +256,12 @@ def main():
         extra["torch_sdpa_bf16_fwd_bwd_ms"] = round(ms_sb, 4)
         extra["torch_sdpa_bf16_fwd_bwd_tflops"] = round((F_fwd + F_bwd) / (ms_sb * 1e-3) / 1e12, 2)
 
-    if args.all_configs:
+    if not args.quick:
         others = {"long_context_B1_H16_N16384_D128_noncausal": (1, 16, 16384, 128, False, "outlier"),
                   "small_head_B16_H16_N2048_D64_causal": (16, 16, 2048, 64, True, "uniform")}
         del q, k, v, do, qq, kq, o, lse
         for name, (b2, h2, n2, d2, c2, dist) in others.items():
-            q2, k2, v2, do2 = (t.to(dev) for t in oracle.make_inputs(dist, b2, h2, n2, d2, seed=0))
+            q2, k2, v2, do2 = (t.to(dev) for t in make_inputs(dist, b2, h2, n2, d2, seed=0))
             sm2 = 1.0 / math.sqrt(d2)
             f2 = flops_fwd(b2, h2, n2, n2, d2, c2)
             qq2, kq2 = qfa.quantize_for_attention(q2), qfa.quantize_for_attention(k2)
@@ -234,7 +273,8 @@ def main():
             extra[name] = {"fwd_ms": round(mf, 4), "fwd_tflops": round(f2 / mf / 1e9, 2), "bwd_ms": round(mb, 4),
                            "bwd_tflops": round(2.5 * f2 / mb / 1e9, 2),
                            "fwd_bwd_tflops": round(3.5 * f2 / (mf + mb) / 1e9, 2),
-                           "quant_ms_per_tensor": round(mq, 4), "quant_GBps": round(qb / mq / 1e6, 1)}
+                           "quant_ms_per_tensor": round(mq, 4), "quant_GBps": round(qb / mq / 1e6, 1),
+                           "quant_frac_hbm_peak": round(qb / mq / 1e6 / PEAK_HBM_GBS, 4)}
             del q2, k2, v2, do2, qq2, kq2, o2, lse2
 
     # ---- roofline of the dominant kernel (attention forward): half its FLOPs are INT8 (QK^T), half
@@ -245,14 +285,15 @@ def main():
     roofline = {"bound": "mfma", "kernel": "fwd_kernel<bf16,128,causal>", "achieved": round(achieved, 2),
                 "peak": round(peak_blend, 1), "unit": "TFLOP/s", "frac": round(achieved / peak_blend, 4),
                 "traffic": FWD_TRAFFIC_BYTES, "algorithmic_flops_per_launch": F_fwd,
-                "mean_launch_ms": round(ms_fwd_kernel, 4),
+                "mean_launch_ms": round(ms_fwd_kernel, 4), "min_launch_ms": round(launch_ms[0], 4),
+                "median_launch_ms": round(launch_ms[len(launch_ms) // 2], 4),
                 "frac_of_bf16_peak": round(achieved / PEAK_BF16_TFLOPS, 4),
                 "peak_note": "harmonic blend of published dense INT8 (5.0 POP/s, QK^T half) and bf16 (2.5 PFLOP/s, PV half)"}
 
     result = {
         "metric": "attn TFLOPS fwd & fwd+bwd @B4 H32 N4096 D128 causal; % of INT8 MFMA peak",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_step, 4), "settle_ms": round(settle_ms, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8 (QK^T, int32 accumulate) + bf16 (P.V) + fp32 softmax", "data": "synthetic",
         "config": {"workload": "forward causal B=4 H=32 N=4096 D=128 bf16: quantize Q, quantize K, attention forward",
                    "flops_convention": "4*B*H*N*N*D/2 (compute_flops.py:103, causal-halved)"},

@@ -182,26 +182,39 @@ def bwd_delta(o: torch.Tensor, do: torch.Tensor, dtype: torch.dtype = torch.floa
     return (o.to(dtype) * do.to(dtype)).sum(-1)
 
 
-def attn_bwd(qh, kh, v, do, causal: bool, sm_scale: float, dtype: torch.dtype = torch.float64):
+def attn_bwd(qh, kh, v, do, causal: bool, sm_scale: float, dtype: torch.dtype = torch.float64,
+             o: Optional[torch.Tensor] = None, spread: bool = False):
     """Closed-form backward of attn_fwd (quant_flash_attn.py:153-164, K and V separate).
 
         P = exp(S - LSE);  dV = P^T dO;  dP = dO V^T;  dS = P o (dP - delta)
         dQ = sm_scale dS K^;  dK = sm_scale dS^T Q^
     Gradients are with respect to the dequantized q^, k^ (straight-through to q, k).
+
+    `o`: the output tensor the forward SAVED, as the reference's backward receives it (quant_flash_attn.py:207-223:
+    delta = rowsum(o * do) is taken from the saved 16-bit o, :97-99).  None: the exact O of these inputs, which makes
+    the result the exact gradient of attn_fwd (what autograd gives).
+    `spread`: also return, per gradient element, the 2-norm of the terms of the sum that forms it
+    (sqrt(sum_j (a_ij b_jd)^2)): the scale of the rounding error any evaluation with 16-bit operands carries.
     """
     q, k, vv, g = qh.to(dtype), kh.to(dtype), v.to(dtype), do.to(dtype)
-    o, lse = attn_fwd(q, k, vv, causal, sm_scale, dtype)
+    o_exact, lse = attn_fwd(q, k, vv, causal, sm_scale, dtype)
     s = (q @ k.transpose(-1, -2)) * sm_scale
     if causal:
         s = s.masked_fill(~_causal_mask(q.shape[-2], k.shape[-2], s.device), float("-inf"))
     p = torch.exp(s - lse[..., None])
     dv = p.transpose(-1, -2) @ g
     dp = g @ vv.transpose(-1, -2)
-    delta = bwd_delta(o, g, dtype)
+    delta = bwd_delta(o_exact if o is None else o, g, dtype)
     ds = p * (dp - delta[..., None])
     dq = (ds @ k) * sm_scale
     dk = (ds.transpose(-1, -2) @ q) * sm_scale
-    return dq, dk, dv
+    if not spread:
+        return dq, dk, dv
+    ds2, p2 = ds * ds, p * p
+    nq = torch.sqrt(ds2 @ (k * k)) * sm_scale
+    nk = torch.sqrt(ds2.transpose(-1, -2) @ (q * q)) * sm_scale
+    nv = torch.sqrt(p2.transpose(-1, -2) @ (g * g))
+    return (dq, dk, dv), (nq, nk, nv)
 
 
 def attn_bwd_autograd(qh, kh, v, do, causal: bool, sm_scale: float, dtype: torch.dtype = torch.float64):
@@ -221,11 +234,16 @@ def legacy_fwd(q, kv_codes, kv_scale, kv_zp, sm_scale: float, dtype: torch.dtype
     return attn_fwd(q.to(dtype), kvh, kvh, False, sm_scale, dtype)
 
 
-def legacy_bwd(q, kv_codes, kv_scale, kv_zp, do, sm_scale: float, dtype: torch.dtype = torch.float64):
-    """quant_flash_attn.py:104-166: returns (dq, dkv) with dkv = dv + sm_scale*dk (:161)."""
+def legacy_bwd(q, kv_codes, kv_scale, kv_zp, do, sm_scale: float, dtype: torch.dtype = torch.float64,
+               o: Optional[torch.Tensor] = None, spread: bool = False):
+    """quant_flash_attn.py:104-166: returns (dq, dkv) with dkv = dv + sm_scale*dk (:161); `o` and `spread` as in
+    attn_bwd (the spread of dkv is that of the two sums together)."""
     kvh = dequantize_per_token(kv_codes, kv_scale, kv_zp, dtype)
-    dq, dk, dv = attn_bwd(q.to(dtype), kvh, kvh, do, False, sm_scale, dtype)
-    return dq, dk + dv
+    if not spread:
+        dq, dk, dv = attn_bwd(q.to(dtype), kvh, kvh, do, False, sm_scale, dtype, o=o)
+        return dq, dk + dv
+    (dq, dk, dv), (nq, nk, nv) = attn_bwd(q.to(dtype), kvh, kvh, do, False, sm_scale, dtype, o=o, spread=True)
+    return (dq, dk + dv), (nq, torch.sqrt(nk * nk + nv * nv))
 
 
 # --------------------------------------------------------------------------- CPU baseline path
@@ -262,40 +280,3 @@ def reference_cpu_path(q, k, v, causal: bool, sm_scale: float, do: Optional[torc
         return o
     o.backward(do.to(torch.float32))
     return o, qh.grad, kh.grad, vf.grad
-
-
-# --------------------------------------------------------------------------- synthetic inputs
-def make_inputs(config: str, B: int, H: int, N: int, D: int, seed: int = 0, dtype=torch.bfloat16):
-    """Synthetic q, k, v, dO with the distributions of the benchmark configurations:
-       'normal'  q,k,v ~ N(0,1)                                            (plumbing case)
-       'offset'  N(0,1) + per-token mean ~ N(0,0.5)   (nonzero zero-points; headline config)
-       'outlier' q,k ~ N(0,1) with ceil(0.01*D) channels per head scaled 20x; v ~ N(0,1)
-       'uniform' q,k ~ U(-3,5); v ~ N(0,1)
-    """
-    g = torch.Generator().manual_seed(seed)
-    shape = (B, H, N, D)
-
-    def randn(*s):
-        return torch.randn(*s, generator=g, dtype=torch.float32)
-
-    if config == "normal":
-        q, k, v = randn(*shape), randn(*shape), randn(*shape)
-    elif config == "offset":
-        q = randn(*shape) + 0.5 * randn(B, H, N, 1)
-        k = randn(*shape) + 0.5 * randn(B, H, N, 1)
-        v = randn(*shape) + 0.5 * randn(B, H, N, 1)
-    elif config == "outlier":
-        q, k, v = randn(*shape), randn(*shape), randn(*shape)
-        n_out = max(1, math.ceil(0.01 * D))
-        for h in range(H):
-            idx = torch.randperm(D, generator=g)[:n_out]
-            q[:, h, :, idx] *= 20.0
-            k[:, h, :, idx] *= 20.0
-    elif config == "uniform":
-        q = torch.rand(*shape, generator=g) * 8.0 - 3.0
-        k = torch.rand(*shape, generator=g) * 8.0 - 3.0
-        v = randn(*shape)
-    else:
-        raise ValueError(config)
-    do = randn(*shape)
-    return tuple(t.to(dtype) for t in (q, k, v, do))

@@ -9,6 +9,7 @@ import torch
 
 from helpers import assert_close, max_abs
 from oracle import oracle
+from quant_flash_attn_amd.synthetic import make_inputs
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -53,7 +54,7 @@ CASES = [
 @pytest.mark.parametrize("B,H,Nq,Nk,D,causal,config,dtype", CASES)
 def test_forward_vs_oracle(qfa, B, H, Nq, Nk, D, causal, config, dtype):
     N = max(Nq, Nk)
-    q, k, v, _ = oracle.make_inputs(config, B, H, N, D, seed=Nq + D, dtype=dtype)
+    q, k, v, _ = make_inputs(config, B, H, N, D, seed=Nq + D, dtype=dtype)
     q, k, v = q[:, :, :Nq].contiguous(), k[:, :, :Nk].contiguous(), v[:, :, :Nk].contiguous()
     sm = 1.0 / math.sqrt(D)
     qq, kq, o, lse = _run(qfa, q, k, v, causal, sm)
@@ -109,7 +110,7 @@ def test_fp32_plumbing_configuration(qfa):
                                                    ("outlier", 1, 16, 16384, 128, False),
                                                    ("uniform", 16, 16, 2048, 64, True)])
 def test_full_size_sampled_heads_and_properties(qfa, config, B, H, N, D, causal):
-    q, k, v, _ = oracle.make_inputs(config, B, H, N, D, seed=0)
+    q, k, v, _ = make_inputs(config, B, H, N, D, seed=0)
     sm = 1.0 / math.sqrt(D)
     qq, kq, o, lse = _run(qfa, q, k, v, causal, sm)
     assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
@@ -140,7 +141,7 @@ def test_full_size_sampled_heads_and_properties(qfa, config, B, H, N, D, causal)
 
 def test_key_permutation_invariance(qfa):
     """Non-causal attention does not depend on the order of the keys."""
-    q, k, v, _ = oracle.make_inputs("offset", 1, 2, 512, 128, seed=3)
+    q, k, v, _ = make_inputs("offset", 1, 2, 512, 128, seed=3)
     sm = 1.0 / math.sqrt(128)
     _, _, o, lse = _run(qfa, q, k, v, False, sm)
     perm = torch.randperm(512, generator=torch.Generator().manual_seed(1))
@@ -149,7 +150,7 @@ def test_key_permutation_invariance(qfa):
 
 
 def test_output_fully_written_and_deterministic(qfa):
-    q, k, v, _ = oracle.make_inputs("normal", 2, 2, 300, 128, seed=8)
+    q, k, v, _ = make_inputs("normal", 2, 2, 300, 128, seed=8)
     sm = 0.1
     qq = qfa.quantize_for_attention(q.to(DEV))
     kq = qfa.quantize_for_attention(k.to(DEV))
@@ -162,7 +163,7 @@ def test_output_fully_written_and_deterministic(qfa):
 def test_strided_qkv_layout(qfa):
     """q, k, v stored [B,N,H,D] and passed as permuted views."""
     B, H, N, D = 2, 3, 256, 64
-    q, k, v, _ = oracle.make_inputs("offset", B, H, N, D, seed=12)
+    q, k, v, _ = make_inputs("offset", B, H, N, D, seed=12)
     mk = lambda t: t.permute(0, 2, 1, 3).contiguous().to(DEV).permute(0, 2, 1, 3)
     o = qfa.quant_flash_attn_qkv(mk(q), mk(k), mk(v), True, 0.125)
     o_c = qfa.quant_flash_attn_qkv(q.to(DEV), k.to(DEV), v.to(DEV), True, 0.125)

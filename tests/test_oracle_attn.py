@@ -12,6 +12,7 @@ import torch
 import torch.nn.functional as F
 
 from oracle import oracle
+from quant_flash_attn_amd.synthetic import make_inputs
 
 
 def _rand(*shape, seed=0, dtype=torch.float64):
@@ -78,7 +79,7 @@ def test_delta_closed_form():
 def test_integer_cross_term_identity(config, D):
     """A - zk*rq - zq*rk + D*zq*zk == sum_d (qc - zq)(kc - zk), exactly, and the dequantized
     dot product equals scale_q * scale_k * that integer."""
-    q, k, _, _ = oracle.make_inputs(config, 1, 2, 96, D, seed=3)
+    q, k, _, _ = make_inputs(config, 1, 2, 96, D, seed=3)
     qc, _, zq, sq, rq = oracle.quantize_per_token(q)
     kc, _, zk, sk, rk = oracle.quantize_per_token(k)
     got = oracle.int_scores(qc, zq, kc, zk)

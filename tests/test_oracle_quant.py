@@ -14,6 +14,7 @@ import pytest
 import torch
 
 from oracle import oracle
+from quant_flash_attn_amd.synthetic import make_inputs
 
 
 from exact_model import quant_row_exact, rn32, roundf_exact  # noqa: F401  (exact model of binary32 arithmetic)
@@ -107,7 +108,7 @@ def test_fp16_scale_is_rne_cast_of_fp32_scale():
 # ---------------------------------------------------------------- invariants on realistic rows
 @pytest.mark.parametrize("config", ["normal", "offset", "outlier", "uniform"])
 def test_invariants(config):
-    q, k, _, _ = oracle.make_inputs(config, 1, 2, 256, 128, seed=1)
+    q, k, _, _ = make_inputs(config, 1, 2, 256, 128, seed=1)
     for x in (q, k):
         codes, _, zp, scale32, rowsum = oracle.quantize_per_token(x)
         xf = x.float()
@@ -127,7 +128,7 @@ def test_invariants(config):
 
 
 def test_c_and_numpy_restatements_agree_on_large_input():
-    q, k, _, _ = oracle.make_inputs("offset", 2, 4, 1024, 128, seed=5)
+    q, k, _, _ = make_inputs("offset", 2, 4, 1024, 128, seed=5)
     for x in (q, k.float() * 3.7):
         n_codes, _, n_zp, n_scale, n_rowsum = oracle.quantize_per_token(x)
         c_codes, c_scale, c_zp, c_rowsum = oracle.quantize_per_token_c(x)
@@ -137,7 +138,7 @@ def test_c_and_numpy_restatements_agree_on_large_input():
 
 def test_torch_eager_baseline_matches_oracle():
     """The torch-eager quantizer that the CPU baseline times gives the oracle's codes."""
-    q, _, _, _ = oracle.make_inputs("uniform", 1, 2, 512, 64, seed=2)
+    q, _, _, _ = make_inputs("uniform", 1, 2, 512, 64, seed=2)
     codes, scale, zp = oracle._quantize_torch_eager(q)
     o_codes, _, o_zp, o_scale, _ = oracle.quantize_per_token(q)
     assert torch.equal(codes, o_codes) and torch.equal(zp, o_zp) and torch.equal(scale, o_scale)

@@ -4,6 +4,7 @@ import pytest
 import torch
 
 from oracle import oracle
+from quant_flash_attn_amd.synthetic import make_inputs
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -31,7 +32,7 @@ def _check(qfa, x_cpu, name=""):
 @pytest.mark.parametrize("D", [32, 64, 128, 256])
 @pytest.mark.parametrize("config", ["normal", "offset", "outlier", "uniform"])
 def test_bit_exact_vs_oracle(qfa, dtype, D, config):
-    q, k, _, _ = oracle.make_inputs(config, 2, 3, 257, D, seed=D, dtype=dtype)   # ragged N
+    q, k, _, _ = make_inputs(config, 2, 3, 257, D, seed=D, dtype=dtype)   # ragged N
     _check(qfa, q, f"{config}/q")
     _check(qfa, k, f"{config}/k")
 
@@ -82,12 +83,12 @@ def test_strided_input(qfa):
 @pytest.mark.parametrize("config,B,H,N,D", [("offset", 4, 32, 4096, 128), ("uniform", 16, 16, 2048, 64)])
 def test_full_size_bit_exact(qfa, config, B, H, N, D):
     """Whole benchmark-size tensors (524 288 tokens) against the C oracle."""
-    q, _, _, _ = oracle.make_inputs(config, B, H, N, D, seed=0)
+    q, _, _, _ = make_inputs(config, B, H, N, D, seed=0)
     _check(qfa, q, f"{config} full size")
 
 
 def test_dequantize_kernel(qfa):
-    q, _, _, _ = oracle.make_inputs("offset", 1, 2, 130, 128, seed=4)
+    q, _, _, _ = make_inputs("offset", 1, 2, 130, 128, seed=4)
     got = qfa.quantize_for_attention(q.to(DEV))
     ref = oracle.dequantize_per_token(got.codes.cpu(), got.scale.cpu(), got.zero_point.cpu())
     out32 = qfa.dequantize_per_token(got.codes, got.scale, got.zero_point, torch.float32)
@@ -98,7 +99,7 @@ def test_dequantize_kernel(qfa):
 
 
 def test_outputs_fully_written_and_deterministic(qfa):
-    q, _, _, _ = oracle.make_inputs("normal", 1, 3, 1000, 64, seed=6)
+    q, _, _, _ = make_inputs("normal", 1, 3, 1000, 64, seed=6)
     xg = q.to(DEV)
     a = qfa.quantize_for_attention(xg)
     b = qfa.quantize_for_attention(xg)

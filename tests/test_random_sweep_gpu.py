@@ -83,13 +83,13 @@ def test_shared_kv_random_sweep(qfa):
         dq, dkv = qfa.attn_bwd_shared_kv(q.to(DEV), codes, scale, zp, o, do.to(DEV), lse, sm)
         c, s_, z = codes.cpu(), scale.cpu(), zp.cpu()
         o_ref, lse_ref = oracle.legacy_fwd(q, c, s_, z, sm)
-        dq_ref, dkv_ref = oracle.legacy_bwd(q, c, s_, z, do, sm)
+        (dq_ref, dkv_ref), (nq, nkv) = oracle.legacy_bwd(q, c, s_, z, do, sm, o=o.cpu(), spread=True)
         case = f"case {it}: {kind} B{B} H{H} Nq{Nq} Nk{Nk} D{D}"
         assert_close(case + " O", o.cpu(), o_ref, scaled=True)
         assert max_abs(lse.cpu(), lse_ref) < 2.0 ** -8 * max(1.0, float(lse_ref.abs().max()) / 64), case
-        one_hot = kind == "ramp" or Nk == 1
-        assert_close(case + " dQ", dq.cpu(), dq_ref, scaled=True, cos_tol=-1 if one_hot else 0.999)
-        assert_close(case + " dKV", dkv.cpu(), dkv_ref, scaled=True)
+        # with a single key P = 1 and dS = 0: dQ is exactly zero and its cosine undefined
+        assert_close(case + " dQ", dq.cpu(), dq_ref, scaled=True, spread=nq, cos_tol=-1 if Nk == 1 else 0.999)
+        assert_close(case + " dKV", dkv.cpu(), dkv_ref, scaled=True, spread=nkv)
         assert torch.isfinite(dq).all() and torch.isfinite(dkv).all(), case
 
 
@@ -120,10 +120,11 @@ def test_backward_random_sweep(qfa):
         dq, dk, dv = qfa.attn_bwd_quantized(qq, kq, v.to(DEV), o, do.to(DEV), lse, causal, sm)
         qh = oracle.dequantize_per_token(qq.codes.cpu(), qq.scale.cpu(), qq.zero_point.cpu(), torch.float64)
         kh = oracle.dequantize_per_token(kq.codes.cpu(), kq.scale.cpu(), kq.zero_point.cpu(), torch.float64)
-        rq, rk, rv = oracle.attn_bwd(qh, kh, v, do, causal, sm)
+        # the closed forms in fp64 on what the kernel is given, the saved 16-bit O included: where softmax rows are
+        # nearly one-hot (ramp, spike, big) dS cancels down to the rounding of that O, for every implementation
+        (rq, rk, rv), (nq, nk, nv) = oracle.attn_bwd(qh, kh, v, do, causal, sm, o=o.cpu(), spread=True)
         case = f"case {it}: {kind} B{B} H{H} Nq{Nq} Nk{Nk} D{D} {dt} causal={causal}"
-        cos = 0.999 if kind == "normal" else -1   # nearly one-hot rows: the rounding of O alone moves small dQ, dK
-        assert_close(case + " dQ", dq.cpu(), rq, scaled=True, cos_tol=cos)
-        assert_close(case + " dK", dk.cpu(), rk, scaled=True, cos_tol=cos)
-        assert_close(case + " dV", dv.cpu(), rv, scaled=True, cos_tol=0.99)
+        assert_close(case + " dQ", dq.cpu(), rq, scaled=True, spread=nq)
+        assert_close(case + " dK", dk.cpu(), rk, scaled=True, spread=nk)
+        assert_close(case + " dV", dv.cpu(), rv, scaled=True, spread=nv)
         assert torch.isfinite(dq).all() and torch.isfinite(dk).all() and torch.isfinite(dv).all(), case

@@ -9,12 +9,13 @@ import pytest
 import torch
 
 from oracle import oracle
+from quant_flash_attn_amd.synthetic import make_inputs
 
 DEV = "cuda:0"
 
 
 def _problem(qfa, B, H, Nq, Nk, D, dtype, seed):
-    q, kv, _, _ = oracle.make_inputs("offset", B, H, max(Nq, Nk), D, seed=seed, dtype=dtype)
+    q, kv, _, _ = make_inputs("offset", B, H, max(Nq, Nk), D, seed=seed, dtype=dtype)
     q, kv = q[:, :, :Nq].contiguous().to(DEV), kv[:, :, :Nk].contiguous().to(DEV)
     codes, scale, zp = qfa.asymmetric_quant_per_token(kv)
     return q, codes, scale.float().reshape(-1).contiguous(), zp.reshape(-1).contiguous()
