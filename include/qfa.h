@@ -56,7 +56,9 @@ const char *qfa_last_error(void);
  *   zp        [B*H*N] int8
  *   rowsum    nullable; [B*H*N] int32 sum of the token's codes (feeds the zero-point
  *             cross term of qfa_attn_fwd / qfa_attn_bwd; not produced by the reference)
- *   D in {32, 64, 128, 256}.  x and codes 16-byte aligned, strides multiples of 16 bytes.
+ *   D any multiple of 8 up to 256 (the reference masks the tail of its power-of-two block the same way,
+ *   asymmetric_quant.py:72-75,97-99).  x 16-byte aligned with strides that are multiples of 16 bytes; codes
+ *   8-byte aligned with strides that are multiples of 8 bytes (the attention entry points want 16).
  * A token row that holds an infinity or a NaN gets unspecified codes (the formulas above send NaN through
  * roundf and the int8 conversion, in the reference as here); the other rows are not affected.
  */

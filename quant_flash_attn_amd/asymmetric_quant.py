@@ -88,7 +88,7 @@ def dequantize_per_token(codes: torch.Tensor, scale: torch.Tensor, zero_point: t
     if dtype not in _lib.DTYPE_CODE or scale.dtype not in _lib.DTYPE_CODE:
         raise TypeError("dtype and scale.dtype must be float16, bfloat16 or float32")
     B, H, N, D = codes.shape
-    if codes.stride(3) != 1 or any(codes.stride(i) % 16 for i in range(3)) or codes.data_ptr() % 16:
+    if codes.stride(3) != 1 or any(codes.stride(i) % 8 for i in range(3)) or codes.data_ptr() % 8:
         codes = codes.contiguous()
     scale = scale.reshape(-1).contiguous()
     zero_point = zero_point.reshape(-1).contiguous()

@@ -27,6 +27,7 @@ int check_launch(const char *what) {
 
 static constexpr int64_t kMaxTokens = 1LL << 28;   // longest sequence (Nq, Nk) the attention entry points take
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static bool aligned8(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
 static bool is_float_dtype(int d) { return d == QFA_F32 || d == QFA_F16 || d == QFA_BF16; }
 static int elem_size(int d) { return d == QFA_F32 ? 4 : 2; }
 
@@ -55,13 +56,13 @@ int qfa_quant_per_token(const void *x, int x_dtype, int8_t *codes, float *scale_
   if (scale_lp && scale_lp_dtype != QFA_F16 && scale_lp_dtype != QFA_BF16)
     return set_error(QFA_EINVAL, "quant: scale_lp_dtype %d is not QFA_F16/BF16", scale_lp_dtype);
   if (B <= 0 || H <= 0 || N <= 0) return set_error(QFA_EINVAL, "quant: B, H, N must be positive");
-  if (D != 32 && D != 64 && D != 128 && D != 256)
-    return set_error(QFA_EUNSUPPORTED, "quant: head_dim %d not in {32, 64, 128, 256}", D);
-  if (!aligned16(x) || !aligned16(codes)) return set_error(QFA_EINVAL, "quant: x and codes must be 16-byte aligned");
+  if (D < 8 || D > 256 || D % 8 != 0)
+    return set_error(QFA_EUNSUPPORTED, "quant: head_dim %d is not a multiple of 8 between 8 and 256", D);
+  if (!aligned16(x) || !aligned8(codes)) return set_error(QFA_EINVAL, "quant: x must be 16-byte, codes 8-byte aligned");
   if (!strides_ok(sxb, sxh, sxn, D, elem_size(x_dtype)))
     return set_error(QFA_EINVAL, "quant: x strides must be positive multiples of 16 bytes, token stride >= D");
-  if (!strides_ok(scb, sch, scn, D, 1) || scn % 8 != 0)
-    return set_error(QFA_EINVAL, "quant: codes strides must be positive multiples of 16 bytes, token stride >= D");
+  if (scb <= 0 || sch <= 0 || scn < D || scb % 8 != 0 || sch % 8 != 0 || scn % 8 != 0)
+    return set_error(QFA_EINVAL, "quant: codes strides must be positive multiples of 8 bytes, token stride >= D");
   return launch_quant(x, x_dtype, codes, scale_f32, scale_lp, scale_lp_dtype, zp, rowsum, B, H, N, D, sxb, sxh, sxn,
                       scb, sch, scn, (hipStream_t)stream);
 }
@@ -73,11 +74,12 @@ int qfa_dequant_per_token(const int8_t *codes, const void *scale, int scale_dtyp
   if (!is_float_dtype(scale_dtype) || !is_float_dtype(out_dtype))
     return set_error(QFA_EINVAL, "dequant: bad scale_dtype/out_dtype");
   if (B <= 0 || H <= 0 || N <= 0) return set_error(QFA_EINVAL, "dequant: B, H, N must be positive");
-  if (D != 32 && D != 64 && D != 128 && D != 256)
-    return set_error(QFA_EUNSUPPORTED, "dequant: head_dim %d not in {32, 64, 128, 256}", D);
-  if (!aligned16(codes) || !aligned16(out)) return set_error(QFA_EINVAL, "dequant: codes and out must be 16-byte aligned");
-  if (!strides_ok(scb, sch, scn, D, 1) || !strides_ok(sob, soh, son, D, elem_size(out_dtype)))
-    return set_error(QFA_EINVAL, "dequant: strides must be positive multiples of 16 bytes, token stride >= D");
+  if (D < 8 || D > 256 || D % 8 != 0)
+    return set_error(QFA_EUNSUPPORTED, "dequant: head_dim %d is not a multiple of 8 between 8 and 256", D);
+  if (!aligned8(codes) || !aligned16(out)) return set_error(QFA_EINVAL, "dequant: codes must be 8-byte, out 16-byte aligned");
+  if (scb <= 0 || sch <= 0 || scn < D || scb % 8 != 0 || sch % 8 != 0 || scn % 8 != 0 ||
+      !strides_ok(sob, soh, son, D, elem_size(out_dtype)))
+    return set_error(QFA_EINVAL, "dequant: strides must be positive, token stride >= D, multiples of 8 bytes (codes) and 16 bytes (out)");
   return launch_dequant(codes, scale, scale_dtype, zp, out, out_dtype, B, H, N, D, scb, sch, scn, sob, soh, son,
                         (hipStream_t)stream);
 }

@@ -7,7 +7,10 @@
 // correctly rounded division and nothing is fused or re-associated: codes and zero points
 // are bit-identical to a CPU evaluation of the same expressions.
 //
-// Mapping: a token of D elements is held by D/8 adjacent lanes (8 elements = one 16-byte
+// Mapping: a token of D elements is held by D/8 adjacent lanes, rounded up to a power of two (head dimensions
+// that are not one leave the group's last lanes idle: they hold a second copy of the token's first eight
+// elements, which changes no minimum or maximum, and neither add to the row sum nor store -- the reference
+// masks its tail lanes the same way, asymmetric_quant.py:72-75,97-99) (8 elements = one 16-byte
 // load per lane for 16-bit inputs, two for fp32), so one wave64 load instruction covers
 // 512/D tokens with fully coalesced 16-byte accesses.  The row is read once, kept in
 // registers, reduced with DPP lane permutes inside the lane group (no LDS), and the codes
@@ -96,14 +99,18 @@ struct QuantArgs {
   int64_t sxb, sxh, sxn, scb, sch, scn;
   int chunks_per_bh;  // ceil(N / tokens per block)
   int scale_lp_dtype;
+  int D;              // head dimension (a multiple of 8, at most the kernel's DP)
 };
 
-// One block = 256 threads = U passes over 256/(D/8) tokens of one (b,h) slice.
-template <typename T, int D, int U> __global__ __launch_bounds__(256) void quant_kernel(QuantArgs a) {
-  constexpr int LPT = D / 8;          // lanes per token
+// One block = 256 threads = U passes over 256/(DP/8) tokens of one (b,h) slice.  DP = the head dimension
+// rounded up to a power of two; PARTIAL: the head dimension is smaller than DP.
+template <typename T, int DP, int U, bool PARTIAL> __global__ __launch_bounds__(256) void quant_kernel(QuantArgs a) {
+  constexpr int LPT = DP / 8;         // lanes per token
   constexpr int TPP = 256 / LPT;      // tokens per pass
   const int tid = threadIdx.x;
   const int sub = tid % LPT;
+  const bool lane_used = !PARTIAL || sub * 8 < a.D;
+  const int sub_ld = lane_used ? sub : 0;   // idle lanes duplicate the token's first eight elements
   const int64_t bh = blockIdx.x / a.chunks_per_bh;
   const int64_t chunk = blockIdx.x % a.chunks_per_bh;
   const int64_t b = bh / a.H, h = bh % a.H;
@@ -118,7 +125,7 @@ template <typename T, int D, int U> __global__ __launch_bounds__(256) void quant
     const int64_t n = n0 + (int64_t)u * TPP;
     live[u] = n < a.N;
     const int64_t nn = live[u] ? n : a.N - 1;   // tail lanes re-read the last token, never store
-    Load8<T>::run(xb + nn * a.sxn + sub * 8, v[u]);
+    Load8<T>::run(xb + nn * a.sxn + sub_ld * 8, v[u]);
   }
 #pragma unroll
   for (int u = 0; u < U; ++u) {
@@ -174,10 +181,11 @@ template <typename T, int D, int U> __global__ __launch_bounds__(256) void quant
     }
     int sum = (int)__builtin_amdgcn_sad_u8(w[0], 0u, 0u);
     sum = (int)__builtin_amdgcn_sad_u8(w[1], 0u, (unsigned)sum) - 8 * 128;
+    if (PARTIAL && !lane_used) sum = 0;
     w[0] ^= 0x80808080u;
     w[1] ^= 0x80808080u;
     sum = group_sum<LPT>(sum);
-    if (live[u]) {
+    if (live[u] && lane_used) {
       *reinterpret_cast<u32x2 *>(cb + n * a.scn + sub * 8) = w;
       if (sub == 0) {
         const int64_t t = bh * a.N + n;
@@ -193,24 +201,27 @@ template <typename T, int D, int U> __global__ __launch_bounds__(256) void quant
   }
 }
 
-template <typename T, int D> static int launch_quant_d(const QuantArgs &a0, int64_t BH, hipStream_t st) {
+template <typename T, int DP> static int launch_quant_d(const QuantArgs &a0, int64_t BH, hipStream_t st) {
   constexpr int U = 4;
-  constexpr int TOK = (256 / (D / 8)) * U;
+  constexpr int TOK = (256 / (DP / 8)) * U;
   QuantArgs a = a0;
   const int64_t chunks = (a.N + TOK - 1) / TOK;
   if (chunks * BH > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "quant: too many tokens for one launch");
   a.chunks_per_bh = (int)chunks;
-  quant_kernel<T, D, U><<<dim3((unsigned)(chunks * BH)), dim3(256), 0, st>>>(a);
+  const dim3 grid((unsigned)(chunks * BH)), block(256);
+  if (a.D == DP) quant_kernel<T, DP, U, false><<<grid, block, 0, st>>>(a);
+  else quant_kernel<T, DP, U, true><<<grid, block, 0, st>>>(a);
   return check_launch("qfa_quant_per_token");
 }
-template <typename T> static int launch_quant_t(const QuantArgs &a, int D, int64_t BH, hipStream_t st) {
-  switch (D) {
+// head dimension rounded up to a power of two (the lane groups the reductions run over), 32 at least
+static int padded_head_dim(int D) { return D <= 32 ? 32 : D <= 64 ? 64 : D <= 128 ? 128 : 256; }
+template <typename T> static int launch_quant_t(const QuantArgs &a, int64_t BH, hipStream_t st) {
+  switch (padded_head_dim(a.D)) {
     case 32: return launch_quant_d<T, 32>(a, BH, st);
     case 64: return launch_quant_d<T, 64>(a, BH, st);
     case 128: return launch_quant_d<T, 128>(a, BH, st);
-    case 256: return launch_quant_d<T, 256>(a, BH, st);
   }
-  return set_error(QFA_EUNSUPPORTED, "quant: head_dim must be 32, 64, 128 or 256");
+  return launch_quant_d<T, 256>(a, BH, st);
 }
 
 int launch_quant(const void *x, int x_dtype, int8_t *codes, float *scale, void *scale_lp, int scale_lp_dtype,
@@ -219,11 +230,12 @@ int launch_quant(const void *x, int x_dtype, int8_t *codes, float *scale, void *
   QuantArgs a;
   a.x = x; a.codes = codes; a.scale = scale; a.scale_lp = scale_lp; a.zp = zp; a.rowsum = rowsum;
   a.N = N; a.H = H; a.sxb = sxb; a.sxh = sxh; a.sxn = sxn; a.scb = scb; a.sch = sch; a.scn = scn;
-  a.chunks_per_bh = 0; a.scale_lp_dtype = scale_lp_dtype;
+  a.chunks_per_bh = 0; a.scale_lp_dtype = scale_lp_dtype; a.D = D;
+  if (D < 8 || D > 256 || D % 8 != 0) return set_error(QFA_EUNSUPPORTED, "quant: head_dim must be a multiple of 8, at most 256");
   switch (x_dtype) {
-    case QFA_F32: return launch_quant_t<float>(a, D, B * H, st);
-    case QFA_F16: return launch_quant_t<_Float16>(a, D, B * H, st);
-    case QFA_BF16: return launch_quant_t<__bf16>(a, D, B * H, st);
+    case QFA_F32: return launch_quant_t<float>(a, B * H, st);
+    case QFA_F16: return launch_quant_t<_Float16>(a, B * H, st);
+    case QFA_BF16: return launch_quant_t<__bf16>(a, B * H, st);
   }
   return set_error(QFA_EINVAL, "quant: bad x_dtype");
 }
@@ -239,10 +251,11 @@ struct DequantArgs {
   int64_t scb, sch, scn, sob, soh, son;
   int chunks_per_bh;
   int scale_dtype;
+  int D;   // head dimension (a multiple of 8, at most the kernel's DP)
 };
 
-template <typename TO, int D> __global__ __launch_bounds__(256) void dequant_kernel(DequantArgs a) {
-  constexpr int LPT = D / 8;
+template <typename TO, int DP> __global__ __launch_bounds__(256) void dequant_kernel(DequantArgs a) {
+  constexpr int LPT = DP / 8;
   constexpr int TPP = 256 / LPT;
   const int tid = threadIdx.x;
   const int sub = tid % LPT;
@@ -250,7 +263,7 @@ template <typename TO, int D> __global__ __launch_bounds__(256) void dequant_ker
   const int64_t chunk = blockIdx.x % a.chunks_per_bh;
   const int64_t b = bh / a.H, h = bh % a.H;
   const int64_t n = chunk * (int64_t)TPP + tid / LPT;
-  if (n >= a.N) return;
+  if (n >= a.N || sub * 8 >= a.D) return;
   const int64_t t = bh * a.N + n;
   float scale;
   if (a.scale_dtype == QFA_F32) scale = reinterpret_cast<const float *>(a.scale)[t];
@@ -278,6 +291,9 @@ template <typename TO, int D> __global__ __launch_bounds__(256) void dequant_ker
 }
 
 template <typename TO> static int launch_dequant_t(DequantArgs a, int D, int64_t BH, hipStream_t st) {
+  if (D < 8 || D > 256 || D % 8 != 0) return set_error(QFA_EUNSUPPORTED, "dequant: head_dim must be a multiple of 8, at most 256");
+  a.D = D;
+  D = padded_head_dim(D);
   const int tpp = 256 / (D / 8);
   const int64_t chunks = (a.N + tpp - 1) / tpp;
   if (chunks * BH > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "dequant: too many tokens for one launch");
@@ -288,7 +304,7 @@ template <typename TO> static int launch_dequant_t(DequantArgs a, int D, int64_t
     case 64: dequant_kernel<TO, 64><<<grid, block, 0, st>>>(a); break;
     case 128: dequant_kernel<TO, 128><<<grid, block, 0, st>>>(a); break;
     case 256: dequant_kernel<TO, 256><<<grid, block, 0, st>>>(a); break;
-    default: return set_error(QFA_EUNSUPPORTED, "dequant: head_dim must be 32, 64, 128 or 256");
+    default: return set_error(QFA_EUNSUPPORTED, "dequant: head_dim must be a multiple of 8, at most 256");
   }
   return check_launch("qfa_dequant_per_token");
 }
@@ -299,7 +315,7 @@ int launch_dequant(const int8_t *codes, const void *scale, int scale_dtype, cons
   DequantArgs a;
   a.codes = codes; a.scale = scale; a.zp = zp; a.out = out; a.N = N; a.H = H;
   a.scb = scb; a.sch = sch; a.scn = scn; a.sob = sob; a.soh = soh; a.son = son;
-  a.chunks_per_bh = 0; a.scale_dtype = scale_dtype;
+  a.chunks_per_bh = 0; a.scale_dtype = scale_dtype; a.D = D;
   switch (out_dtype) {
     case QFA_F32: return launch_dequant_t<float>(a, D, B * H, st);
     case QFA_F16: return launch_dequant_t<_Float16>(a, D, B * H, st);

@@ -37,7 +37,9 @@ def test_argument_errors_need_no_gpu(qfa):
     rc = L.qfa_quant_per_token(ok_ptr, 7, ok_ptr, ok_ptr, None, 0, ok_ptr, None, 1, 1, 8, 64, 512, 512, 64, 512, 512, 64, None)
     assert rc == -1 and b"x_dtype" in L.qfa_last_error()
     # unsupported head_dim
-    rc = L.qfa_quant_per_token(ok_ptr, 2, ok_ptr, ok_ptr, None, 0, ok_ptr, None, 1, 1, 8, 48, 384, 384, 48, 384, 384, 48, None)
+    rc = L.qfa_quant_per_token(ok_ptr, 2, ok_ptr, ok_ptr, None, 0, ok_ptr, None, 1, 1, 8, 44, 384, 384, 48, 384, 384, 48, None)
+    assert rc == -2 and b"head_dim" in L.qfa_last_error()
+    rc = L.qfa_quant_per_token(ok_ptr, 2, ok_ptr, ok_ptr, None, 0, ok_ptr, None, 1, 1, 8, 264, 4096, 4096, 264, 4096, 4096, 264, None)
     assert rc == -2 and b"head_dim" in L.qfa_last_error()
     # misaligned pointer, bad stride
     rc = L.qfa_quant_per_token(ok_ptr + 2, 2, ok_ptr, ok_ptr, None, 0, ok_ptr, None, 1, 1, 8, 64, 512, 512, 64, 512, 512, 64, None)

@@ -37,6 +37,21 @@ def test_bit_exact_vs_oracle(qfa, dtype, D, config):
     _check(qfa, k, f"{config}/k")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("D", [8, 40, 96, 136, 200, 248])
+def test_any_head_dim_that_is_a_multiple_of_eight(qfa, dtype, D):
+    """The reference handles any HEAD_DIM by masking the tail of its power-of-two block (asymmetric_quant.py:72-75,
+    97-99); here the lanes past the row hold a copy of its first elements.  Bit-exact codes, zero points, scales and
+    row sums, and the dequantizer on the same widths."""
+    config = "offset" if D % 16 else "uniform"
+    q, _, _, _ = make_inputs(config, 2, 3, 131, D, seed=D, dtype=dtype)
+    got = _check(qfa, q, f"D={D}")
+    from quant_flash_attn_amd import dequantize_per_token
+    back = dequantize_per_token(got.codes, got.scale, got.zero_point, torch.float32).cpu()
+    want = oracle.dequantize_per_token(got.codes.cpu(), got.scale.cpu(), got.zero_point.cpu(), torch.float32)
+    assert torch.equal(back, want.reshape(back.shape))
+
+
 def test_ties_saturation_and_constant_rows(qfa):
     rows = torch.zeros(8, 64)
     rows[0, :8] = torch.tensor([0.0, 255.0, 0.5, 1.5, 2.5, 128.5, 129.5, 130.5])   # exact .5 ties, scale 1
