@@ -359,6 +359,37 @@ def test_shared_kv_graph_capture_and_replay(qfa, B, H, Nq, Nk):
                 assert torch.equal(a_, b_), f"graph replay differs from eager: {name} (round {rep})"
 
 
+def test_shared_kv_full_reference_test_shape(qfa):
+    """The reference's largest accuracy shape at FULL size (test_accuracy.py:44: Z=99, H=53, 97 queries, 689 keys,
+    head_dim 128; 5247 (batch, head) pairs): the forward runs 7 workgroups of 16 queries per pair, the backward its dQ
+    and dKV kernels with their key-chunk plan at a large pair count.  Sampled pairs against the dense fp64 oracle,
+    determinism, and a zero dO giving exactly zero gradients."""
+    Z, H, Nq, Nk, D = 99, 53, 97, 689, 128
+    g = torch.Generator(device=DEV).manual_seed(20)
+    q = torch.randn((Z, H, Nq, D), generator=g, device=DEV, dtype=torch.float16)
+    kv = torch.randn((Z, H, Nk, D), generator=g, device=DEV, dtype=torch.float16)
+    do = torch.randn((Z, H, Nq, D), generator=g, device=DEV, dtype=torch.float16)
+    sm = 1.0 / math.sqrt(D)
+    codes, scale, zp = qfa.asymmetric_quant_per_token(kv)
+    del kv
+    o, lse = qfa.attn_fwd_shared_kv(q, codes, scale, zp, sm)
+    dq, dkv = qfa.attn_bwd_shared_kv(q, codes, scale, zp, o, do, lse, sm)
+    dq2, dkv2 = qfa.attn_bwd_shared_kv(q, codes, scale, zp, o, do, lse, sm)
+    dq0, dkv0 = qfa.attn_bwd_shared_kv(q, codes, scale, zp, o, torch.zeros_like(do), lse, sm)
+    torch.cuda.synchronize()
+    assert torch.equal(dq, dq2) and torch.equal(dkv, dkv2)
+    assert float(dq0.abs().max()) == 0.0 and float(dkv0.abs().max()) == 0.0
+    assert torch.isfinite(o.float()).all() and torch.isfinite(dq.float()).all() and torch.isfinite(dkv.float()).all()
+    for b, h in ((0, 0), (41, 17), (98, 52)):
+        sl = lambda t: t[b:b + 1, h:h + 1].cpu()
+        o_ref, lse_ref = oracle.legacy_fwd(sl(q), sl(codes), sl(scale), sl(zp), sm)
+        (dq_ref, dkv_ref), (nq, nkv) = oracle.legacy_bwd(sl(q), sl(codes), sl(scale), sl(zp), sl(do), sm, o=sl(o), spread=True)
+        assert_close(f"O[{b},{h}]", sl(o), o_ref, scaled=True)
+        assert max_abs(sl(lse), lse_ref) < LSE_TOL
+        assert_close(f"dQ[{b},{h}]", sl(dq), dq_ref, scaled=True, spread=nq)
+        assert_close(f"dKV[{b},{h}]", sl(dkv), dkv_ref, scaled=True, spread=nkv)
+
+
 @pytest.mark.parametrize("D", [128, 64])
 def test_shared_kv_full_benchmark_size(qfa, D):
     """The reference's benchmark shape at full size (compute_flops.py:96: Z=512, H=16, 16 queries, 3000 keys):
