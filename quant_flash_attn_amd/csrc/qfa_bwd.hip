@@ -430,18 +430,9 @@ __global__ __launch_bounds__(DqShape<D>::THREADS, DqShape<D>::WAVES_PER_SIMD) vo
     __syncthreads();
   }
 
-  if (qi < a.Nq) {
-    T *row = dq_bh + (int64_t)qi * a.sdqn;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int aa = 0; aa < 4; ++aa) {
-        u32x2 w;
-        w[0] = pack2<T>(dqacc[db][4 * aa + 0] * a.sm_scale, dqacc[db][4 * aa + 1] * a.sm_scale);
-        w[1] = pack2<T>(dqacc[db][4 * aa + 2] * a.sm_scale, dqacc[db][4 * aa + 3] * a.sm_scale);
-        *reinterpret_cast<u32x2 *>(row + 32 * db + 8 * aa + 4 * g) = w;
-      }
-  }
+  // dQ leaves as whole rows through LDS (the tile buffers are free after the last barrier)
+  static_assert((DQ_THREADS / 64) * 32 * 2 * D <= 2 * BUF, "output staging fits the tile buffers");
+  store_tile_rows<T, D>(dqacc, a.sm_scale, smem + (tid / 64) * (32 * 2 * D), dq_bh, a.sdqn, q_first, a.Nq, tid % 64);
 }
 
 // ------------------------------------------------------------------------------------------ dK, dV
@@ -783,19 +774,12 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
     }
   }
 
-  if (kj < a.Nk) {
-    T *row = (p_role ? dv_bh + (int64_t)kj * a.sdvn : dk_bh + (int64_t)kj * a.sdkn);
-    const float scale = p_role ? 1.0f : a.sm_scale;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int aa = 0; aa < 4; ++aa) {
-        u32x2 w;
-        w[0] = pack2<T>(oacc[db][4 * aa + 0] * scale, oacc[db][4 * aa + 1] * scale);
-        w[1] = pack2<T>(oacc[db][4 * aa + 2] * scale, oacc[db][4 * aa + 3] * scale);
-        *reinterpret_cast<u32x2 *>(row + 32 * db + 8 * aa + 4 * g) = w;
-      }
-  }
+  // dK / dV leave as whole rows through LDS: a barrier first, the last block's exchange slots and fragments may
+  // still be read by the partner waves
+  __syncthreads();
+  static_assert((DKV_THREADS / 64) * 32 * 2 * D <= 2 * BUF + NP * 4096, "output staging fits the workgroup's LDS");
+  if (p_role) store_tile_rows<T, D>(oacc, 1.0f, smem + (tid / 64) * (32 * 2 * D), dv_bh, a.sdvn, k_first, a.Nk, tid % 64);
+  else store_tile_rows<T, D>(oacc, a.sm_scale, smem + (tid / 64) * (32 * 2 * D), dk_bh, a.sdkn, k_first, a.Nk, tid % 64);
 }
 
 template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStream_t st) {

@@ -237,6 +237,36 @@ template <int N> __device__ __forceinline__ void lds_wait_async(u32x2 (&r)[8]) {
 template <int N> __device__ __forceinline__ void lds_wait_async(u32x2 (&r)[4]) {
   asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]) : "n"(N) : "memory");
 }
+// A wave's 32 x D result tile, held as the transposed accumulators of the 32x32 MFMAs (lane l: row l%32, register
+// quad aa of block db: columns 32db + 8aa + 4(l/32) + {0..3}), scaled, rounded to T and written to rows
+// row0 .. row0+31 (those below nrows) of a row-major tensor.  Stored directly, one instruction would write 16 bytes
+// to each of 32 rows; the tile goes through `stage` (32 * 2D bytes of LDS owned by this wave, not in use by anybody
+// else) and leaves as whole rows, 16 bytes per lane.  Chunks are XORed with the row so that the 32 rows of one LDS
+// write spread over the banks.
+template <typename T, int D>
+__device__ __forceinline__ void store_tile_rows(const f32x16 (&acc)[D / 32], float scale, unsigned char *stage,
+                                                T *base, int64_t row_stride, int row0, int nrows, int lane) {
+  constexpr int ROWB = 2 * D, CPR = ROWB / 16;
+  asm volatile("" : "+v"(lane));   // addresses are formed here, not hoisted above the caller's main loop
+  const int lr = lane % 32, g = lane / 32;
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int aa = 0; aa < 4; ++aa) {
+      u32x2 w;
+      w[0] = pack2<T>(acc[db][4 * aa + 0] * scale, acc[db][4 * aa + 1] * scale);
+      w[1] = pack2<T>(acc[db][4 * aa + 2] * scale, acc[db][4 * aa + 3] * scale);
+      *reinterpret_cast<u32x2 *>(stage + lr * ROWB + (((4 * db + aa) ^ (lr % CPR)) * 16) + 8 * g) = w;
+    }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave reads back only what it wrote itself
+#pragma unroll
+  for (int i = 0; i < 32 * CPR / 64; ++i) {
+    const int p = lane + 64 * i, row = p / CPR, c = p % CPR;
+    const u32x4 w = *reinterpret_cast<const u32x4 *>(stage + row * ROWB + ((c ^ (row % CPR)) * 16));
+    if (row0 + row < nrows) *reinterpret_cast<u32x4 *>(base + (int64_t)(row0 + row) * row_stride + c * 8) = w;
+  }
+}
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
 // global access, including direct-to-LDS loads issued for a LATER tile, which would serialise the
 // prefetch; this one leaves them in flight (pair it with dma_wait() where a tile must have landed).

@@ -528,35 +528,10 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
   }
   const float l_tot = l_run + swap32_f(l_run);
   const float inv = 1.0f / l_tot;
-  // The accumulators hold O^T: a lane has 4 consecutive d of ONE query per register quad, so stored directly a
-  // wave instruction writes 16 bytes to each of 32 rows.  The wave's 32 x D tile goes through LDS instead (all
-  // tile buffers are free after the last barrier; 32 * 2D bytes per wave at the start of the K area) and leaves
-  // as whole rows: 16 bytes per lane, four 2D-byte rows per instruction.
-  {
-    constexpr int ROWB = 2 * D;                       // bytes per row
-    unsigned char *stage = smem + wave * (32 * ROWB);
-    static_assert(FWD_WAVES * 32 * ROWB <= SM::OFF_V + 2 * SM::V_BYTES, "output staging fits the tile buffers");
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int aa = 0; aa < 4; ++aa) {
-        u32x2 w;
-        w[0] = pack2<T>(oacc[db][4 * aa + 0] * inv, oacc[db][4 * aa + 1] * inv);
-        w[1] = pack2<T>(oacc[db][4 * aa + 2] * inv, oacc[db][4 * aa + 3] * inv);
-        // chunk index XORed with the row so that the 32 rows of one instruction spread over the banks
-        const int chunk = (4 * db + aa) ^ (lr % (ROWB / 16));
-        *reinterpret_cast<u32x2 *>(stage + lr * ROWB + chunk * 16 + 8 * g) = w;
-      }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave reads back only what it wrote itself
-    constexpr int CPR = ROWB / 16;                     // 16-byte chunks per row
-#pragma unroll
-    for (int i = 0; i < 32 * CPR / 64; ++i) {
-      const int p = lane + 64 * i, row = p / CPR, c = p % CPR;
-      const u32x4 w = *reinterpret_cast<const u32x4 *>(stage + row * ROWB + ((c ^ (row % CPR)) * 16));
-      const int qrow = m0 + wave * 32 + row;
-      if (qrow < a.Nq) *reinterpret_cast<u32x4 *>(o_bh + (int64_t)qrow * a.son + c * 8) = w;
-    }
-  }
+  // O leaves as whole rows through LDS (all tile buffers are free after the last barrier; every wave takes 32 * 2D
+  // bytes at the start of the K area)
+  static_assert(FWD_WAVES * 32 * 2 * D <= SM::OFF_V + 2 * SM::V_BYTES, "output staging fits the tile buffers");
+  store_tile_rows<T, D>(oacc, inv, smem + wave * (32 * 2 * D), o_bh, a.son, m0 + wave * 32, a.Nq, lane);
   if (qi < a.Nq && g == 0) a.lse[tq0 + qi] = (a_i * m_ref + __log2f(l_tot)) * kLn2;
 }
 
