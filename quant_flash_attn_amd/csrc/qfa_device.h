@@ -109,9 +109,10 @@ __device__ __forceinline__ float max_across_halves(float x) {
 // chosen so that 16 consecutive rows read at the same logical chunk hit 16 different 16-byte slots
 // of the 256-byte bank line.
 template <int ROW_BYTES> struct Swz {
-  static constexpr int CPR = ROW_BYTES / 16;                 // chunks per row (4, 8 or 16)
-  static constexpr int RP = 16 / CPR;                        // rows per 256 bytes
-  static __device__ __forceinline__ int swz(int row) { return (row / RP) % CPR; }
+  static constexpr int CPR = ROW_BYTES / 16;                 // chunks per row (4, 8, 16 or 32)
+  static constexpr int RP = CPR >= 16 ? 1 : 16 / CPR;        // rows per 256 bytes (1 for rows of one or more lines)
+  static constexpr int MOD = CPR >= 16 ? 16 : CPR;           // only the slot inside the 256-byte line matters
+  static __device__ __forceinline__ int swz(int row) { return (row / RP) % MOD; }
   // byte offset of logical chunk c of row r inside the tile
   static __device__ __forceinline__ int off(int r, int c) { return r * ROW_BYTES + ((c ^ swz(r)) << 4); }
 };
@@ -132,7 +133,7 @@ typedef __attribute__((address_space(3))) void *lptr_t;
 template <int ROW_BYTES> struct SwzQuad {
   static constexpr int CPR = ROW_BYTES / 16;
   static constexpr int RPL = ROW_BYTES >= 256 ? 1 : 256 / ROW_BYTES;   // rows per 256-byte line
-  static constexpr int QPR = ROW_BYTES / 64;                             // 64-byte quarters per row
+  static constexpr int QPR = ROW_BYTES >= 256 ? 4 : ROW_BYTES / 64;      // quarters the XOR moves over (one line at most)
   static __device__ __forceinline__ int swz(int row) { return 4 * ((row / RPL) % QPR); }
 };
 
@@ -231,6 +232,13 @@ template <int OFF> __device__ __forceinline__ u32x2 lds_read_tr16_async(unsigned
 template <int N> __device__ __forceinline__ void lds_wait_async(u32x2 (&r)[8]) {
   asm volatile("s_waitcnt lgkmcnt(%8)"
                : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7])
+               : "n"(N)
+               : "memory");
+}
+template <int N> __device__ __forceinline__ void lds_wait_async(u32x2 (&r)[16]) {
+  asm volatile("s_waitcnt lgkmcnt(%16)"
+               : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]),
+                 "+v"(r[8]), "+v"(r[9]), "+v"(r[10]), "+v"(r[11]), "+v"(r[12]), "+v"(r[13]), "+v"(r[14]), "+v"(r[15])
                : "n"(N)
                : "memory");
 }

@@ -52,7 +52,7 @@ namespace qfa {
 // (it writes the scaled row maximum where the LSE would go and leaves O untouched).  It exists to
 // time the QK^T stage by itself against the INT8 MFMA peak.
 template <typename T, int D, bool CAUSAL, bool QK_ONLY = false, int NW = FWD_WAVES>
-__global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
+__global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(FwdArgs a) {
   constexpr int NT = 64 * NW;        // threads per workgroup
   constexpr int FWD_BM = 32 * NW;    // queries per workgroup
   typedef FwdSmem<D> SM;
@@ -109,10 +109,18 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
   // query side of the rank-4 correction: k-group 0 multiplies the two digits of rk by -zq,
   // k-group 1 multiplies zk (stored twice) by minus the two digits of c = rq - D*zq
   u32x4 corr_q = {0u, 0u, 0u, 0u};
-  {
+  if (D <= 128) {
     const int c = a.rq[tq0 + qi_c] - D * zq_i;     // |c| <= 32640
     const int hi = c >> 7, lo = c & 127;
     corr_q[0] = g == 0 ? pack2<T>((float)(-zq_i), (float)(-zq_i)) : pack2<T>((float)(-128 * hi), (float)(-lo));
+  } else {
+    // head_dim 256: rq - D*zq no longer splits into two digits of 8 bits, so k-group 1 carries three terms against
+    // (zk, zk, zk): minus the two digits of rq, and D*zq (a multiple of 256 below 2^15: exact).  The key side puts
+    // the same dword in both slots; k-group 0 multiplies its second copy by zero.
+    const int rq = a.rq[tq0 + qi_c];
+    const int hi = rq >> 7, lo = rq & 127;
+    corr_q[0] = g == 0 ? pack2<T>((float)(-zq_i), (float)(-zq_i)) : pack2<T>((float)(-128 * hi), (float)(-lo));
+    corr_q[1] = g == 0 ? 0u : pack2<T>((float)(D * zq_i), 0.0f);
   }
   const int q_first = m0 + wave * 32, q_last = q_first + 31;
 
@@ -214,7 +222,8 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
     f32x16 f;
 #pragma unroll
     for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
-    u32x4 corr_k = {dgp[2 * (32 * nb + lr) + g], 0u, 0u, 0u};
+    const unsigned dg = dgp[2 * (32 * nb + lr) + g];
+    const u32x4 corr_k = {dg, D <= 128 ? 0u : dg, 0u, 0u};
     f = mfma_16b<T>(corr_k, corr_q, f);
     float mt = -INFINITY;
 #pragma unroll
@@ -370,7 +379,7 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
     // `copy(i)`, i = 0..2, is called between phases: the steady loop issues chunks of the next
     // tiles' copies there, so that the memory pipe sees a few requests at a time instead of a burst per tile
     auto body = [&](int vbuf, auto nb_tag, int cbuf, int cnb, int kbuf, int knb, auto &&copy) {
-      static_assert(DB == 4 || DB == 2, "fragment arrays are sized for head_dim 128 or 64");
+      static_assert(DB == 8 || DB == 4 || DB == 2, "fragment arrays are sized for head_dim 256, 128 or 64");
       u32x2 vr0[2 * DB], vr1[2 * DB];
       u32x4 pf0, pf1;
       i32x16 s;
@@ -396,14 +405,15 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
       if (!QK_ONLY) {
         check_half(0, pf0, l0);
         v_frags(vbuf, NB, std::integral_constant<int, 1>{}, vr1);
-        lds_wait_async<2 * DB>(vr0);   // the 2*DB requests just made may still be in flight
+        lds_wait_async<(2 * DB < 15 ? 2 * DB : 15)>(vr0);   // the 2*DB requests just made may still be in flight (the counter holds 15)
       }
       const unsigned char *cb = smem + SM::OFF_C + cbuf * SM::C_BYTES;
       f32x4 sk4[4];
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa)
         sk4[aa] = *reinterpret_cast<const f32x4 *>(cb + (32 * cnb + 8 * aa + 4 * g) * 4);
-      const u32x4 corr_k = {reinterpret_cast<const unsigned *>(cb + FWD_BN * 4)[2 * (32 * cnb + lr) + g], 0u, 0u, 0u};
+      const unsigned dg = reinterpret_cast<const unsigned *>(cb + FWD_BN * 4)[2 * (32 * cnb + lr) + g];
+      const u32x4 corr_k = {dg, D <= 128 ? 0u : dg, 0u, 0u};
       __builtin_amdgcn_sched_barrier(0);
       // P.V of the first 16 keys under the exponentials of the second 16 and the conversion of the next
       // block's raw scores; their zero-point correction (one MFMA) goes last, so that its result has the
@@ -478,12 +488,12 @@ __global__ __launch_bounds__(64 * NW, 2) void fwd_kernel(FwdArgs a) {
         if (i < KCH) cp_k.issue_one(rs_k, kd, wave_u, tid, i);
         else if (i < KCH + VCH) cp_v.issue_one(rs_v, vd, wave_u, tid, i - KCH);
       };
+      constexpr int PER = (KCH + VCH + 2) / 3;   // chunks per slot: 2 at head_dim 128, 4 at 256
       body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, [&](auto i) {
-        chunk(2 * decltype(i)::value);
-        chunk(2 * decltype(i)::value + 1);
+#pragma unroll
+        for (int c = 0; c < PER; ++c) chunk(PER * decltype(i)::value + c);
       });
       body(t & 1, std::integral_constant<int, 1>{}, kb_nxt, 0, kb_nxt, 1, no_copy);
-      static_assert(KCH + VCH <= 6, "six copy slots per tile");
       store_k(kb_free);
       const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
       dma_wait();
@@ -568,15 +578,17 @@ template <typename T, int D> static int launch_fwd_td(const AttnArgs &x, hipStre
 
 int launch_fwd(const AttnArgs &x, hipStream_t st, bool qk_only) {
   if (x.io_dtype == QFA_BF16) {
+    if (x.D == 256) return launch_fwd_td<__bf16, 256>(x, st, qk_only);
     if (x.D == 128) return launch_fwd_td<__bf16, 128>(x, st, qk_only);
     if (x.D == 64) return launch_fwd_td<__bf16, 64>(x, st, qk_only);
   } else if (x.io_dtype == QFA_F16) {
+    if (x.D == 256) return launch_fwd_td<_Float16, 256>(x, st, qk_only);
     if (x.D == 128) return launch_fwd_td<_Float16, 128>(x, st, qk_only);
     if (x.D == 64) return launch_fwd_td<_Float16, 64>(x, st, qk_only);
   } else {
     return set_error(QFA_EINVAL, "attn_fwd: io_dtype must be QFA_BF16 or QFA_F16");
   }
-  return set_error(QFA_EUNSUPPORTED, "attn_fwd: head_dim must be 64 or 128");
+  return set_error(QFA_EUNSUPPORTED, "attn_fwd: head_dim must be 64, 128 or 256");
 }
 
 }  // namespace qfa

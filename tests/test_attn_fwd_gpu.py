@@ -48,6 +48,13 @@ CASES = [
     # a partial group at the end
     (3, 4, 320, 320, 64, True, "normal", torch.bfloat16),
     (1, 19, 300, 300, 128, True, "offset", torch.bfloat16),
+    # head_dim 256 (compute_flops.py:94): one workgroup per CU, three-term zero-point correction
+    (1, 2, 256, 256, 256, False, "normal", torch.bfloat16),
+    (2, 3, 384, 384, 256, True, "offset", torch.bfloat16),
+    (1, 2, 1024, 1024, 256, True, "outlier", torch.float16),
+    (1, 2, 333, 333, 256, True, "uniform", torch.bfloat16),     # ragged, causal
+    (2, 2, 97, 689, 256, False, "offset", torch.float16),       # short Q, long ragged KV
+    (1, 3, 700, 700, 256, False, "uniform", torch.bfloat16),
 ]
 
 
@@ -66,7 +73,7 @@ def test_forward_vs_oracle(qfa, B, H, Nq, Nk, D, causal, config, dtype):
     assert torch.equal(qq.codes.cpu(), oracle.quantize_per_token_c(q)[0])
 
 
-@pytest.mark.parametrize("D,dtype", [(128, torch.bfloat16), (64, torch.float16)])
+@pytest.mark.parametrize("D,dtype", [(128, torch.bfloat16), (64, torch.float16), (256, torch.bfloat16)])
 @pytest.mark.parametrize("jump", [64, 80, 104, 352])
 @pytest.mark.parametrize("causal", [False, True])
 def test_scores_jump_far_above_the_running_reference(qfa, D, dtype, jump, causal):
