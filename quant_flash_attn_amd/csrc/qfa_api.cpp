@@ -84,7 +84,7 @@ int qfa_dequant_per_token(const int8_t *codes, const void *scale, int scale_dtyp
                         (hipStream_t)stream);
 }
 
-static int check_attn_common(const char *who, const AttnArgs &a, bool d256 = true) {
+static int check_attn_common(const char *who, const AttnArgs &a) {
   if (!a.qc || !a.sq || !a.zq || !a.rq || !a.kc || !a.sk || !a.zk || !a.rk || !a.v || !a.o || !a.lse)
     return set_error(QFA_EINVAL, "%s: null pointer argument", who);
   if (a.io_dtype != QFA_BF16 && a.io_dtype != QFA_F16)
@@ -93,8 +93,8 @@ static int check_attn_common(const char *who, const AttnArgs &a, bool d256 = tru
   // the kernels form byte offsets into the per-token vectors (4 bytes per token) in 31 bits
   if (a.Nq > kMaxTokens || a.Nk > kMaxTokens)
     return set_error(QFA_EUNSUPPORTED, "%s: sequences of more than 2^28 tokens are not supported", who);
-  if (a.D != 64 && a.D != 128 && !(d256 && a.D == 256))
-    return set_error(QFA_EUNSUPPORTED, "%s: head_dim %d not in {64, 128%s}", who, a.D, d256 ? ", 256" : "");
+  if (a.D != 64 && a.D != 128 && a.D != 256)
+    return set_error(QFA_EUNSUPPORTED, "%s: head_dim %d not in {64, 128, 256}", who, a.D);
   if (!(a.sm_scale > 0.0f) || !(a.sm_scale < 3.0e38f))
     return set_error(QFA_EINVAL, "%s: sm_scale must be a positive finite number", who);
   if (a.causal && a.Nq != a.Nk) return set_error(QFA_EUNSUPPORTED, "%s: causal needs Nq == Nk", who);
@@ -248,7 +248,7 @@ int qfa_bwd_delta(const void *o, const void *dout, float *delta, int io_dtype, i
   if (!o || !dout || !delta) return set_error(QFA_EINVAL, "bwd_delta: null pointer argument");
   if (io_dtype != QFA_BF16 && io_dtype != QFA_F16) return set_error(QFA_EINVAL, "bwd_delta: io_dtype must be QFA_BF16 or QFA_F16");
   if (B <= 0 || H <= 0 || N <= 0) return set_error(QFA_EINVAL, "bwd_delta: B, H, N must be positive");
-  if (D != 64 && D != 128) return set_error(QFA_EUNSUPPORTED, "bwd_delta: head_dim %d not in {64, 128}", D);
+  if (D != 64 && D != 128 && D != 256) return set_error(QFA_EUNSUPPORTED, "bwd_delta: head_dim %d not in {64, 128, 256}", D);
   if (!aligned16(o) || !aligned16(dout)) return set_error(QFA_EINVAL, "bwd_delta: o and dout must be 16-byte aligned");
   if (!strides_ok(sob, soh, son, D, 2) || !strides_ok(sdb, sdh, sdn, D, 2))
     return set_error(QFA_EINVAL, "bwd_delta: strides must be positive multiples of 16 bytes, token stride >= D");
@@ -256,7 +256,7 @@ int qfa_bwd_delta(const void *o, const void *dout, float *delta, int io_dtype, i
 }
 
 int64_t qfa_attn_bwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D) {
-  if (B <= 0 || H <= 0 || Nq <= 0 || Nk <= 0 || (D != 64 && D != 128)) return 0;
+  if (B <= 0 || H <= 0 || Nq <= 0 || Nk <= 0 || (D != 64 && D != 128 && D != 256)) return 0;
   return bwd_workspace_bytes(B, H, Nq, Nk, D);
 }
 
@@ -280,7 +280,7 @@ int qfa_attn_bwd(const int8_t *qc, const float *sq, const int8_t *zq, const int3
   a.sdob = sdob; a.sdoh = sdoh; a.sdon = sdon; a.sdqb = sdqb; a.sdqh = sdqh; a.sdqn = sdqn;
   a.sdkb = sdkb; a.sdkh = sdkh; a.sdkn = sdkn; a.sdvb = sdvb; a.sdvh = sdvh; a.sdvn = sdvn;
   a.sm_scale = sm_scale; a.causal = causal;
-  if (int e = check_attn_common("attn_bwd", a, false)) return e;
+  if (int e = check_attn_common("attn_bwd", a)) return e;
   if (!dout || !workspace || !dq || !dk || !dv) return set_error(QFA_EINVAL, "attn_bwd: null pointer argument");
   if (!aligned16(dout) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv) || !aligned16(workspace))
     return set_error(QFA_EINVAL, "attn_bwd: dout, dq, dk, dv, workspace must be 16-byte aligned");

@@ -59,6 +59,7 @@ template <typename T, int D> __global__ __launch_bounds__(256) void delta_kernel
   s += dpp_f<0x4E>(s);
   s += dpp_f<0x141>(s);
   if (LPT >= 16) s += dpp_f<0x140>(s);
+  if (LPT >= 32) s += __shfl_xor(s, 16);
   if (n < a.N && sub == 0) a.delta[bh * a.N + n] = s;
 }
 
@@ -73,32 +74,37 @@ int launch_delta(const void *o, const void *dout, float *delta, int io_dtype, in
   a.chunks_per_bh = (int)chunks;
   const dim3 grid((unsigned)(chunks * B * H)), block(256);
   if (io_dtype == QFA_BF16) {
-    if (D == 128) delta_kernel<__bf16, 128><<<grid, block, 0, st>>>(a);
+    if (D == 256) delta_kernel<__bf16, 256><<<grid, block, 0, st>>>(a);
+    else if (D == 128) delta_kernel<__bf16, 128><<<grid, block, 0, st>>>(a);
     else delta_kernel<__bf16, 64><<<grid, block, 0, st>>>(a);
   } else {
-    if (D == 128) delta_kernel<_Float16, 128><<<grid, block, 0, st>>>(a);
+    if (D == 256) delta_kernel<_Float16, 256><<<grid, block, 0, st>>>(a);
+    else if (D == 128) delta_kernel<_Float16, 128><<<grid, block, 0, st>>>(a);
     else delta_kernel<_Float16, 64><<<grid, block, 0, st>>>(a);
   }
   return check_launch("qfa_bwd_delta");
 }
 
 // ------------------------------------------------------------------------------------------ shared
-constexpr int BWD_TILE = 64;   // rows streamed per step
-
-// Workspace layout: per (batch*head, 64-query tile) a Q-side blob, then per (batch*head, 64-key tile)
-// a K-side blob.  Transposed tiles are [D][64] 16-bit values, 128-byte rows, positions permuted.
+// Rows streamed per step: 64, or 32 at head_dim 256, where a 64-row step of codes, 16-bit rows and transposed tile
+// (80 KB) could not be double-buffered in a CU's 160 KB.
+// Workspace layout: per (batch*head, query tile) a Q-side blob, then per (batch*head, key tile)
+// a K-side blob.  Transposed tiles are [D][TILE] 16-bit values (128- or 64-byte rows), positions permuted.
 template <int D> struct BwdWs {
-  static constexpr int T_BYTES = D * BWD_TILE * 2;            // one transposed tile
-  static constexpr int CQ_BYTES = 5 * BWD_TILE * 4;           // digits (2 dwords/query), a, -lse*log2e, -delta
-  static constexpr int CK_BYTES = 3 * BWD_TILE * 4;           // digits (2 dwords/key), key scale
+  static constexpr int TILE = D > 128 ? 32 : 64;
+  static constexpr int CSH = D > 128 ? 8 : 7;             // bits per digit of rq - D*zq (|.| <= 65280 at head_dim 256)
+  static constexpr int T_BYTES = D * TILE * 2;            // one transposed tile
+  static constexpr int CQ_BYTES = 5 * TILE * 4;           // digits (2 dwords/query), a, -lse*log2e, -delta
+  static constexpr int CK_BYTES = 3 * TILE * 4;           // digits (2 dwords/key), key scale
   static constexpr int Q_BLOB = T_BYTES + CQ_BYTES;           // Qz^T, constants
   static constexpr int K_BLOB = T_BYTES + CK_BYTES;           // Kz^T, constants
 };
 
 int64_t bwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D) {
-  const int64_t tq = (Nq + BWD_TILE - 1) / BWD_TILE, tk = (Nk + BWD_TILE - 1) / BWD_TILE;
-  const int64_t qb = D == 128 ? BwdWs<128>::Q_BLOB : BwdWs<64>::Q_BLOB;
-  const int64_t kb = D == 128 ? BwdWs<128>::K_BLOB : BwdWs<64>::K_BLOB;
+  const int64_t tile = D == 256 ? BwdWs<256>::TILE : 64;
+  const int64_t tq = (Nq + tile - 1) / tile, tk = (Nk + tile - 1) / tile;
+  const int64_t qb = D == 256 ? BwdWs<256>::Q_BLOB : D == 128 ? BwdWs<128>::Q_BLOB : BwdWs<64>::Q_BLOB;
+  const int64_t kb = D == 256 ? BwdWs<256>::K_BLOB : D == 128 ? BwdWs<128>::K_BLOB : BwdWs<64>::K_BLOB;
   return B * H * (tq * qb + tk * kb);
 }
 
@@ -119,7 +125,7 @@ struct BwdArgs {
   int group_log2;       // causal: log2 of the number of heads whose blocks are dispatched together (set per launch)
 };
 
-// position of streamed row r (0..63) inside a transposed tile: the order in which the 32x32
+// position of streamed row r (0..63, or 0..31 in a 32-row tile) inside a transposed tile: the order in which the 32x32
 // accumulator layout hands out rows to a lane (two runs of 4 per 16-row MFMA k-slice)
 __device__ __forceinline__ int perm_pos4(int r4) {   // r4 = r / 4
   return 32 * (r4 / 8) + 16 * ((r4 / 4) % 2) + 8 * (r4 % 2) + 4 * ((r4 / 2) % 2);
@@ -141,16 +147,18 @@ __device__ __forceinline__ void store_codes_transposed(const u32x2 (&c)[4], cons
     *reinterpret_cast<u32x2 *>(dst + e * stride) = o;
   }
 }
-// integer n -> (128*floor(n/128), n mod 128) resp. their negatives, as a packed pair of 16-bit floats
-template <typename T> __device__ __forceinline__ unsigned base128_pair(int n, float sign) {
-  const int hi = n >> 7, lo = n & 127;
-  return pack2<T>(sign * (float)(hi * 128), sign * (float)lo);
+// integer n -> (2^SH * floor(n / 2^SH), n mod 2^SH) resp. their negatives, as a packed pair of 16-bit floats
+template <typename T, int SH = 7> __device__ __forceinline__ unsigned base128_pair(int n, float sign) {
+  const int hi = n >> SH, lo = n & ((1 << SH) - 1);
+  return pack2<T>(sign * (float)(hi * (1 << SH)), sign * (float)lo);
 }
 
 // ------------------------------------------------------------------------------------------ prep
 // One block per (b,h, 64-query tile): delta, Qz^T and the per-query constants.
 template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_q_kernel(BwdArgs a) {
   typedef BwdWs<D> WS;
+  constexpr int BWD_TILE = WS::TILE;
+  static_assert((BWD_TILE / 4) * (D / 8) <= 256, "one thread per 4 rows x 8 columns");
   __shared__ float red[D / 8][BWD_TILE];
   const int tid = threadIdx.x;
   const int bh = blockIdx.x / a.tiles_q, tile = blockIdx.x % a.tiles_q;
@@ -158,7 +166,7 @@ template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_q_k
   const int i0 = tile * BWD_TILE;
   const int64_t tq0 = (int64_t)bh * a.Nq;
   unsigned char *blob = a.ws_q + ((int64_t)bh * a.tiles_q + tile) * WS::Q_BLOB;
-  const int r4 = tid % 16, dc = tid / 16;
+  const int r4 = tid % (BWD_TILE / 4), dc = tid / (BWD_TILE / 4);
   if (dc < D / 8) {
     const int8_t *qc_bh = a.qc + b * a.sqb + h * a.sqh;
     const T *do_bh = reinterpret_cast<const T *>(a.dout) + b * a.sdob + h * a.sdoh;
@@ -197,7 +205,7 @@ template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_q_k
     unsigned *cq = reinterpret_cast<unsigned *>(blob + WS::T_BYTES);
     u32x2 dg;
     dg[0] = pack2<T>((float)(-zq), (float)(-zq));      // k-group 0: times the two digits of rk
-    dg[1] = base128_pair<T>(c, -1.0f);                 // k-group 1: minus the digits of rq - D*zq, times zk
+    dg[1] = base128_pair<T, WS::CSH>(c, -1.0f);        // k-group 1: minus the digits of rq - D*zq, times zk
     reinterpret_cast<u32x2 *>(cq)[tid] = dg;
     reinterpret_cast<float *>(cq)[2 * BWD_TILE + tid] = a.sq[tq0 + i] * a.sm_scale_log2;
     reinterpret_cast<float *>(cq)[3 * BWD_TILE + tid] = -a.lse[tq0 + i] * kLog2e;
@@ -208,13 +216,14 @@ template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_q_k
 // One block per (b,h, 64-key tile): Kz^T and the per-key constants.
 template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_k_kernel(BwdArgs a) {
   typedef BwdWs<D> WS;
+  constexpr int BWD_TILE = WS::TILE;
   const int tid = threadIdx.x;
   const int bh = blockIdx.x / a.tiles_k, tile = blockIdx.x % a.tiles_k;
   const int64_t b = bh / a.H, h = bh % a.H;
   const int j0 = tile * BWD_TILE;
   const int64_t tk0 = (int64_t)bh * a.Nk;
   unsigned char *blob = a.ws_k + ((int64_t)bh * a.tiles_k + tile) * WS::K_BLOB;
-  const int r4 = tid % 16, dc = tid / 16;
+  const int r4 = tid % (BWD_TILE / 4), dc = tid / (BWD_TILE / 4);
   if (dc < D / 8) {
     const int8_t *kc_bh = a.kc + b * a.skb + h * a.skh;
     u32x2 creg[4];
@@ -246,9 +255,10 @@ template <typename T, int D> __global__ __launch_bounds__(256) void bwd_prep_k_k
 // 8 waves = 256 queries, one workgroup per CU (two 41 KB tile buffers).  D=64: the loop fits 170 registers
 // and the buffers 42 KB, so three workgroups of 4 waves run per CU (3 waves per SIMD; backward of
 // B16 H16 N2048 D64 causal 0.90 -> 0.84 ms against 8-wave workgroups, 2-wave ones are slower again).
+// D=256: 4 waves, one per SIMD (128 accumulators, 96 operand registers), two 41 KB buffers of 32-key tiles.
 template <int D> struct DqShape {
-  static constexpr int THREADS = D == 64 ? 256 : 512;
-  static constexpr int WAVES_PER_SIMD = D == 64 ? 3 : 2;
+  static constexpr int THREADS = D == 128 ? 512 : 256;
+  static constexpr int WAVES_PER_SIMD = D == 64 ? 3 : D == 128 ? 2 : 1;
   static constexpr int BLK = 32 * (THREADS / 64);
 };
 
@@ -256,6 +266,7 @@ template <typename T, int D, bool CAUSAL>
 __global__ __launch_bounds__(DqShape<D>::THREADS, DqShape<D>::WAVES_PER_SIMD) void bwd_dq_kernel(BwdArgs a) {
   constexpr int DQ_THREADS = DqShape<D>::THREADS, DQ_BLK = DqShape<D>::BLK;
   typedef BwdWs<D> WS;
+  constexpr int BWD_TILE = WS::TILE, NBLK = BWD_TILE / 32;
   typedef Swz<D> SK;            // K code rows
   typedef Swz<2 * D> SV;        // V rows
   typedef Swz<BWD_TILE * 2> ST; // transposed rows
@@ -416,10 +427,10 @@ __global__ __launch_bounds__(DqShape<D>::THREADS, DqShape<D>::WAVES_PER_SIMD) vo
   for (int t = 0; t < ntiles; ++t) {
     const int j0 = t * BWD_TILE;
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
+    for (int nb = 0; nb < NBLK; ++nb) {
       if (t + 1 < ntiles) {
         if (nb == 0) load_tile_a(t + 1);
-        else load_tile_b(t + 1);
+        if (nb == NBLK - 1) load_tile_b(t + 1);
       }
       const int jb = j0 + 32 * nb;
       if ((jb >= a.Nk) || (CAUSAL && jb > q_last)) continue;               // wave-uniform
@@ -453,9 +464,10 @@ __global__ __launch_bounds__(DqShape<D>::THREADS, DqShape<D>::WAVES_PER_SIMD) vo
 // SIMD (the loop takes 220 registers).  D=64: 6 pairs, 3 waves per SIMD (145 registers); backward of
 // B16 H16 N2048 D64 causal 0.84 -> 0.805 ms against 4 pairs; 3 pairs with two workgroups per CU are slower
 // (0.95 ms), 8 pairs need 128 registers and spill.
+// D=256: 2 pairs, one wave per SIMD (128 accumulators and up to 200 operand registers), 32-query tiles.
 template <int D> struct DkvShape {
-  static constexpr int PAIRS = D == 64 ? 6 : 4;
-  static constexpr int WAVES_PER_SIMD = D == 64 ? 3 : 2;
+  static constexpr int PAIRS = D == 64 ? 6 : D == 128 ? 4 : 2;
+  static constexpr int WAVES_PER_SIMD = D == 64 ? 3 : D == 128 ? 2 : 1;
   static constexpr int THREADS = 128 * PAIRS, BLK = 32 * PAIRS;
 };
 
@@ -475,6 +487,7 @@ template <typename T, int D, bool CAUSAL>
 __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) void bwd_dkdv_kernel(BwdArgs a) {
   constexpr int NP = DkvShape<D>::PAIRS, DKV_THREADS = DkvShape<D>::THREADS;
   typedef BwdWs<D> WS;
+  constexpr int BWD_TILE = WS::TILE, NBLK = BWD_TILE / 32;
   typedef Swz<D> SQ;            // Q code rows
   typedef SwzDual<2 * D> SG;    // dO rows: read row-wise for dP and through transposing reads for dV
   typedef Swz<BWD_TILE * 2> ST; // transposed rows
@@ -591,8 +604,8 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
   const unsigned t_off = (unsigned)((4 * g + t_row) * (2 * D) +
                                     ((((SG::quarter(t_row)) << 2) | ((2 * ((lane / 16) % 2) + (lane % 4) / 2) ^ g)) << 4) +
                                     8 * (lane % 2));   // XOR 64*db: d block; XOR 32 with +8 rows: the second four queries
-  auto p_first = [&](const unsigned char *base, int i0, int mbk, u32x4 (&pf)[2], u32x2 (&ta)[2 * DB], u32x2 (&tb)[2 * DB],
-                     auto masked_tag) {
+  auto p_first = [&](const unsigned char *base, int i0, int mbk, int slot, u32x4 (&pf)[2], u32x2 (&ta)[2 * DB],
+                     u32x2 (&tb)[2 * DB], auto masked_tag) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     const unsigned *dgp = reinterpret_cast<const unsigned *>(base + OFF_C);
     const float *cs = reinterpret_cast<const float *>(base + OFF_C);
@@ -636,7 +649,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
     for (int hh = 0; hh < 2; ++hh) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) pf[hh][e] = pack2<T>(pp[8 * hh + 2 * e], pp[8 * hh + 2 * e + 1]);
-      xch0[mbk * 128 + hh * 64 + lane] = pf[hh];
+      xch0[slot * 128 + hh * 64 + lane] = pf[hh];
     }
     __builtin_amdgcn_sched_barrier(0);
     // requested behind the compiler's back; the barrier that follows waits for every LDS operation of the
@@ -682,10 +695,10 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
       for (int db = 0; db < DB; ++db) oacc[db] = mfma_16b<T>(tf[hh * DB + db], bf[hh], oacc[db]);
   };
   // ---- dS role, second half prologue: dS = P (from partner) * (dP - delta), packed (dp holds dP - delta)
-  auto ds_second = [&](int mbk, const f32x16 &dp, u32x4 (&dsf)[2]) {
+  auto ds_second = [&](int slot, const f32x16 &dp, u32x4 (&dsf)[2]) {
     u32x4 pw[2];
 #pragma unroll
-    for (int hh = 0; hh < 2; ++hh) pw[hh] = xch0[mbk * 128 + hh * 64 + lane];
+    for (int hh = 0; hh < 2; ++hh) pw[hh] = xch0[slot * 128 + hh * 64 + lane];
     float ds[16];
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh)
@@ -702,6 +715,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
   };
 
   if (it0 < ntiles) load_tile(it0);
+  if (NBLK == 1 && it0 + 1 < ntiles) load_tile(it0 + 1);
   dma_wait();
   __syncthreads();
   // The two roles run separate loops with the same barrier sequence (one per 32-query block).
@@ -710,31 +724,46 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
     on = (ib < a.Nq) && (!CAUSAL || ib + 31 >= k_first);                               // wave-uniform
     masked = (CAUSAL && ib < k_last) || (ib + 32 > a.Nq) || (k_last >= a.Nk);
   };
-  // Block (t, mbk): first phase | barrier | second phase.  The next tile's copy goes out in two halves
-  // around the barrier of the tile's first block and must have landed before the barrier of its
-  // second block (its buffer was last read before the previous tile's last barrier).
+  // Block (t, mbk): first phase | barrier | second phase; all reads of the tile buffers happen in first phases.
+  // 64-query tiles (two blocks): the next tile's copy goes out in two halves around the barrier of the tile's first
+  // block and must have landed before the barrier of its second block (its buffer was last read before the
+  // previous tile's last barrier).  32-query tiles (one block): after the block's barrier nobody reads the tile's
+  // buffer any more, so the tile after the next one is copied into it right there and must have landed before the
+  // next block's barrier.
+  auto before_first = [&](int t, int mbk) {
+    if (NBLK == 2 && mbk == 0 && t + 1 < ntiles) {
+      load_part(t + 1, 0);
+      load_part(t + 1, 1);
+    }
+  };
+  auto barrier = [&](int mbk) {
+    if (mbk == NBLK - 1) dma_wait();
+    lds_barrier();   // P of this block is in LDS
+  };
+  auto after_barrier = [&](int t, int mbk) {
+    if (NBLK == 2) {
+      if (mbk == 0 && t + 1 < ntiles) load_part(t + 1, 2);
+    } else if (t + 2 < ntiles) {
+      load_tile(t + 2);
+    }
+  };
   if (p_role) {
     for (int t = it0; t < ntiles; ++t) {
       const unsigned char *base = smem + (t & 1) * BUF;
 #pragma unroll
-      for (int mbk = 0; mbk < 2; ++mbk) {
-        if (mbk == 0 && t + 1 < ntiles) {
-          load_part(t + 1, 0);
-          load_part(t + 1, 1);
-        }
+      for (int mbk = 0; mbk < NBLK; ++mbk) {
+        const int slot = NBLK == 2 ? mbk : (t & 1);
+        before_first(t, mbk);
         bool on, masked;
         block_flags(t, mbk, on, masked);
         u32x4 pf[2];
         u32x2 ta[2 * DB], tb[2 * DB];
         if (on) {
-          if (masked) p_first(base, t * BWD_TILE, mbk, pf, ta, tb, std::true_type{});
-          else p_first(base, t * BWD_TILE, mbk, pf, ta, tb, std::false_type{});
+          if (masked) p_first(base, t * BWD_TILE, mbk, slot, pf, ta, tb, std::true_type{});
+          else p_first(base, t * BWD_TILE, mbk, slot, pf, ta, tb, std::false_type{});
         }
-        if (mbk == 1) dma_wait();
-        lds_barrier();   // P of this block is in LDS
-        if (mbk == 0 && t + 1 < ntiles) {
-          load_part(t + 1, 2);
-        }
+        barrier(mbk);
+        after_barrier(t, mbk);
         if (on) {
           lds_wait_async<0>(ta);
           lds_wait_async<0>(tb);
@@ -751,23 +780,18 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
     for (int t = it0; t < ntiles; ++t) {
       const unsigned char *base = smem + (t & 1) * BUF;
 #pragma unroll
-      for (int mbk = 0; mbk < 2; ++mbk) {
-        if (mbk == 0 && t + 1 < ntiles) {
-          load_part(t + 1, 0);
-          load_part(t + 1, 1);
-        }
+      for (int mbk = 0; mbk < NBLK; ++mbk) {
+        const int slot = NBLK == 2 ? mbk : (t & 1);
+        before_first(t, mbk);
         bool on, masked;
         block_flags(t, mbk, on, masked);
         u32x4 dsf[2], tf[2 * DB];
         f32x16 dp;
         if (on) ds_first(base, mbk, dp, tf);
-        if (mbk == 1) dma_wait();
-        lds_barrier();
-        if (mbk == 0 && t + 1 < ntiles) {
-          load_part(t + 1, 2);
-        }
+        barrier(mbk);
+        after_barrier(t, mbk);
         if (on) {
-          ds_second(mbk, dp, dsf);
+          ds_second(slot, dp, dsf);
           accumulate(tf, dsf);
         }
       }
@@ -788,8 +812,8 @@ template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStre
   a.qc = x.qc; a.sq = x.sq; a.zq = x.zq; a.rq = x.rq; a.kc = x.kc; a.sk = x.sk; a.zk = x.zk; a.rk = x.rk;
   a.v = x.v; a.o = x.o; a.dout = x.dout; a.lse = x.lse; a.dq = x.dq; a.dk = x.dk; a.dv = x.dv;
   a.H = x.H; a.Nq = (int)x.Nq; a.Nk = (int)x.Nk;
-  a.tiles_q = (int)((x.Nq + BWD_TILE - 1) / BWD_TILE);
-  a.tiles_k = (int)((x.Nk + BWD_TILE - 1) / BWD_TILE);
+  a.tiles_q = (int)((x.Nq + WS::TILE - 1) / WS::TILE);
+  a.tiles_k = (int)((x.Nk + WS::TILE - 1) / WS::TILE);
   a.ws_q = reinterpret_cast<unsigned char *>(x.workspace);
   a.ws_k = a.ws_q + x.B * x.H * (int64_t)a.tiles_q * WS::Q_BLOB;
   a.sqb = x.sqb; a.sqh = x.sqh; a.sqn = x.sqn; a.skb = x.skb; a.skh = x.skh; a.skn = x.skn;
@@ -849,15 +873,17 @@ template <typename T, int D> static int launch_bwd_td(const AttnArgs &x, hipStre
 
 int launch_bwd(const AttnArgs &x, hipStream_t st) {
   if (x.io_dtype == QFA_BF16) {
+    if (x.D == 256) return launch_bwd_td<__bf16, 256>(x, st);
     if (x.D == 128) return launch_bwd_td<__bf16, 128>(x, st);
     if (x.D == 64) return launch_bwd_td<__bf16, 64>(x, st);
   } else if (x.io_dtype == QFA_F16) {
+    if (x.D == 256) return launch_bwd_td<_Float16, 256>(x, st);
     if (x.D == 128) return launch_bwd_td<_Float16, 128>(x, st);
     if (x.D == 64) return launch_bwd_td<_Float16, 64>(x, st);
   } else {
     return set_error(QFA_EINVAL, "attn_bwd: io_dtype must be QFA_BF16 or QFA_F16");
   }
-  return set_error(QFA_EUNSUPPORTED, "attn_bwd: head_dim must be 64 or 128");
+  return set_error(QFA_EUNSUPPORTED, "attn_bwd: head_dim must be 64, 128 or 256");
 }
 
 }  // namespace qfa

@@ -142,10 +142,10 @@ template <int ROW_BYTES> struct SwzQuad {
 // contiguous bytes).  The row's low bits move the 64-byte quarter, bits 2-3 the chunk inside the quarter, so
 // either pattern lands on 16 different 16-byte slots of the 256-byte bank line.
 template <int ROW_BYTES> struct SwzDual {
-  static_assert(ROW_BYTES == 256 || ROW_BYTES == 128, "rows of 128 or 64 16-bit floats");
+  static_assert(ROW_BYTES == 512 || ROW_BYTES == 256 || ROW_BYTES == 128, "rows of 256, 128 or 64 16-bit floats");
   static constexpr int CPR = ROW_BYTES / 16;
   // the part of the XOR that moves quarters (a function of the row's low bits only)
-  static __device__ __forceinline__ int quarter(int row) { return ROW_BYTES == 256 ? (row & 3) : ((row >> 1) & 1); }
+  static __device__ __forceinline__ int quarter(int row) { return ROW_BYTES >= 256 ? (row & 3) : ((row >> 1) & 1); }
   static __device__ __forceinline__ int swz(int row) { return (quarter(row) << 2) | ((row >> 2) & 3); }
   static __device__ __forceinline__ int off(int r, int c) { return r * ROW_BYTES + ((c ^ swz(r)) << 4); }
 };

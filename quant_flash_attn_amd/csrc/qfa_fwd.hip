@@ -18,7 +18,7 @@
 //
 // Zero points.  With integer codes,  sum_d (qc-zq)(kc-zk) = A - zq*rk - zk*(rq - D*zq), A the int32
 // MFMA result and rq, rk the code row sums.  The correction is a rank-4 update with integer
-// entries below 2^8 (rk and rq - D*zq split into base-128 digits), so it runs as ONE extra 16-bit
+// entries of at most 8 significant bits (rk and rq - D*zq split into two digits), so it runs as ONE extra 16-bit
 // MFMA on the converted accumulator instead of per-score VALU work; every product and partial sum
 // is an integer below 2^24, hence exact in fp32.  Then one multiply by the key scale; the query
 // scale, sm_scale and log2(e) are folded into the exp2 argument.
@@ -109,18 +109,13 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   // query side of the rank-4 correction: k-group 0 multiplies the two digits of rk by -zq,
   // k-group 1 multiplies zk (stored twice) by minus the two digits of c = rq - D*zq
   u32x4 corr_q = {0u, 0u, 0u, 0u};
-  if (D <= 128) {
-    const int c = a.rq[tq0 + qi_c] - D * zq_i;     // |c| <= 32640
-    const int hi = c >> 7, lo = c & 127;
-    corr_q[0] = g == 0 ? pack2<T>((float)(-zq_i), (float)(-zq_i)) : pack2<T>((float)(-128 * hi), (float)(-lo));
-  } else {
-    // head_dim 256: rq - D*zq no longer splits into two digits of 8 bits, so k-group 1 carries three terms against
-    // (zk, zk, zk): minus the two digits of rq, and D*zq (a multiple of 256 below 2^15: exact).  The key side puts
-    // the same dword in both slots; k-group 0 multiplies its second copy by zero.
-    const int rq = a.rq[tq0 + qi_c];
-    const int hi = rq >> 7, lo = rq & 127;
-    corr_q[0] = g == 0 ? pack2<T>((float)(-zq_i), (float)(-zq_i)) : pack2<T>((float)(-128 * hi), (float)(-lo));
-    corr_q[1] = g == 0 ? 0u : pack2<T>((float)(D * zq_i), 0.0f);
+  {
+    // two digits of 7 bits each (|c| <= 32640) up to head_dim 128, of 8 bits at head_dim 256 (|c| <= 65280): either
+    // way each digit, shifted into place, has at most 8 significant bits and is exact in the 16-bit type
+    constexpr int SH = D > 128 ? 8 : 7;
+    const int c = a.rq[tq0 + qi_c] - D * zq_i;
+    const int hi = c >> SH, lo = c & ((1 << SH) - 1);
+    corr_q[0] = g == 0 ? pack2<T>((float)(-zq_i), (float)(-zq_i)) : pack2<T>((float)(-(hi * (1 << SH))), (float)(-lo));
   }
   const int q_first = m0 + wave * 32, q_last = q_first + 31;
 
@@ -222,8 +217,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
     f32x16 f;
 #pragma unroll
     for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
-    const unsigned dg = dgp[2 * (32 * nb + lr) + g];
-    const u32x4 corr_k = {dg, D <= 128 ? 0u : dg, 0u, 0u};
+    u32x4 corr_k = {dgp[2 * (32 * nb + lr) + g], 0u, 0u, 0u};
     f = mfma_16b<T>(corr_k, corr_q, f);
     float mt = -INFINITY;
 #pragma unroll
@@ -412,8 +406,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa)
         sk4[aa] = *reinterpret_cast<const f32x4 *>(cb + (32 * cnb + 8 * aa + 4 * g) * 4);
-      const unsigned dg = reinterpret_cast<const unsigned *>(cb + FWD_BN * 4)[2 * (32 * cnb + lr) + g];
-      const u32x4 corr_k = {dg, D <= 128 ? 0u : dg, 0u, 0u};
+      const u32x4 corr_k = {reinterpret_cast<const unsigned *>(cb + FWD_BN * 4)[2 * (32 * cnb + lr) + g], 0u, 0u, 0u};
       __builtin_amdgcn_sched_barrier(0);
       // P.V of the first 16 keys under the exponentials of the second 16 and the conversion of the next
       // block's raw scores; their zero-point correction (one MFMA) goes last, so that its result has the

@@ -55,6 +55,13 @@ CASES = [
     (3, 4, 320, 320, 64, True, "normal", torch.bfloat16),
     (1, 19, 300, 300, 128, True, "offset", torch.bfloat16),
     (2, 8, 512, 512, 64, True, "uniform", torch.float16),
+    # head_dim 256: 32-row tiles, one wave per SIMD
+    (1, 2, 128, 128, 256, False, "normal", torch.bfloat16),
+    (2, 3, 384, 384, 256, True, "offset", torch.bfloat16),
+    (1, 2, 512, 512, 256, True, "outlier", torch.float16),
+    (1, 2, 333, 333, 256, True, "uniform", torch.bfloat16),     # ragged, causal
+    (2, 2, 97, 689, 256, False, "offset", torch.float16),       # short Q, long ragged KV
+    (1, 3, 200, 200, 256, False, "uniform", torch.bfloat16),    # ragged
 ]
 
 
