@@ -87,7 +87,8 @@ int qfa_dequant_per_token(const int8_t *codes, const void *scale, int scale_dtyp
  * separate K and V, a causal flag (rule of flash_attn_triton.py:50) and tiled queries.
  *   qc,kc  int8 [B,H,Nq|Nk,D];  sq,sk float, zq,zk int8, rq,rk int32: dense [B*H*Nq|Nk]
  *   v, o   [B,H,Nk|Nq,D] of io_dtype (QFA_BF16 or QFA_F16);  lse float [B*H*Nq]
- *   D in {64, 128}.  causal != 0 requires Nq == Nk.  All tensors 16-byte aligned, strides
+ *   D in {64, 128, 256} (the widths compute_flops.py:94 sweeps; also for qfa_attn_bwd and qfa_bwd_delta).
+ *   causal != 0 requires Nq == Nk.  All tensors 16-byte aligned, strides
  *   multiples of 16 bytes, token strides below 2^23 elements, Nq and Nk at most 2^28
  *   (QFA_EUNSUPPORTED otherwise).
  */

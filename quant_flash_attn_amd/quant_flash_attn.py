@@ -10,7 +10,7 @@ Two autograd entry points, both backed by the HIP kernels behind qfa_attn_fwd / 
   QuantFlashAttention.apply(q, kv_fp16, kv_quant, sm_scale)     (alias quant_flash_attn)
       The reference's own entry point (quant_flash_attn.py:173-240): one quantized tensor serves as
       K and V, `kv_fp16` only receives the gradient, backward returns (dq, dkv, None, None) with
-      dkv = dK + dV (:161).  Query blocks of up to SHARED_KV_MAX_Q (512) tokens (any length at head_dim 256) run the reference's
+      dkv = dK + dV (:161).  Query blocks of up to SHARED_KV_MAX_Q (512; 1024 at head_dim 256) tokens run the reference's
       computation itself in the forward (Q in 16-bit, qfa_attn_fwd_shared_kv) and in the backward
       (qfa_attn_bwd_shared_kv, binary16 arithmetic; bf16 tensors are converted around it).  Longer
       query blocks go through the INT8-score kernels, where Q is quantized per token too (stated
@@ -125,6 +125,14 @@ def attn_bwd_quantized(qq: QuantizedTokens, kq: QuantizedTokens, v: torch.Tensor
 # benchmark shapes; measured crossover with the INT8-score kernels at Nk=4096, D=128: between 512 and
 # 1024 queries (fwd 1.16 vs 1.51 ms at 512, 1.14 vs 1.01 ms at 1024).
 SHARED_KV_MAX_Q = 512
+# head_dim 256 (compute_flops.py:94): the INT8-score kernels run one wave per SIMD there and the crossover moves up
+# (Nk=4096: fwd+bwd 5.9 vs 4.5 ms at 512 queries, 9.0 vs 8.9 at 1024; Nq=Nk=2048: 3.9 vs 4.9 ms, INT8-score first).
+SHARED_KV_MAX_Q_BY_HEAD_DIM = {256: 1024}   # head_dim -> limit, where it differs from SHARED_KV_MAX_Q
+
+
+def shared_kv_max_q(head_dim: int) -> int:
+    """Longest query block that `quant_flash_attn` gives to the shared-KV kernels at this head_dim."""
+    return SHARED_KV_MAX_Q_BY_HEAD_DIM.get(head_dim, SHARED_KV_MAX_Q)
 
 
 def attn_fwd_shared_kv(q: torch.Tensor, codes: torch.Tensor, scale: torch.Tensor, zero_point: torch.Tensor,
@@ -263,8 +271,7 @@ class QuantFlashAttention(torch.autograd.Function):
             raise ValueError(f"shape mismatch: q {tuple(q.shape)}, kv {tuple(kv_fp16.shape)}, codes {tuple(codes.shape)}")
         ctx.sm_scale = float(sm_scale)
         ctx.q_dtype, ctx.kv_dtype = q.dtype, kv_fp16.dtype
-        # head_dim 256 (compute_flops.py:94) exists only in the shared-KV kernels: any Nq goes there
-        ctx.shared_kv = (q.shape[2] <= SHARED_KV_MAX_Q or q.shape[3] == 256) and q.dtype in _IO_DTYPES
+        ctx.shared_kv = q.shape[2] <= shared_kv_max_q(q.shape[3]) and q.dtype in _IO_DTYPES
         if ctx.shared_kv:
             # the reference's computation itself: Q unquantized, the codes streamed once (:50-69)
             o, lse = attn_fwd_shared_kv(q, codes, scale, zp, sm_scale)

@@ -67,6 +67,12 @@ def test_argument_errors_need_no_gpu(qfa):
     assert rc == -2 and b"2^28" in L.qfa_last_error()
     rc = L.qfa_bwd_delta(None, ok_ptr, ok_ptr, 2, 1, 1, 8, 64, 512, 512, 64, 512, 512, 64, None)
     assert rc == -1
+    # backward scratch: one blob per 64-row tile (32-row at head_dim 256) and side; nothing for other widths
+    ws = L.qfa_attn_bwd_workspace_bytes
+    assert ws(1, 1, 64, 64, 64) == 2 * 64 * 64 * 2 + (5 + 3) * 64 * 4
+    assert ws(2, 3, 65, 64, 128) == 6 * (3 * 128 * 64 * 2 + (2 * 5 + 3) * 64 * 4)
+    assert ws(1, 1, 64, 32, 256) == 3 * 256 * 32 * 2 + (2 * 5 + 3) * 32 * 4
+    assert ws(1, 1, 64, 64, 96) == 0 and ws(1, 1, 0, 64, 64) == 0
     # shared-KV entry points
     def skv_fwd(Nq=16, Nk=100, D=128, io=1, sdt=1, sm=0.1, q=ok_ptr):
         sq, sc = (Nq * D, Nq * D, D), (Nk * D, Nk * D, D)

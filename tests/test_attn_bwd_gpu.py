@@ -78,14 +78,48 @@ def test_backward_vs_oracle(qfa, B, H, Nq, Nk, D, causal, config, dtype):
     _check_grads("", (dq.cpu(), dk.cpu(), dv.cpu()), want, spreads)
 
 
-def test_delta_kernel(qfa):
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_extreme_row_sums_and_zero_points(qfa, D):
+    """Rows that sit entirely at one end of their range: zero point -128 with codes near +127 and zero point +127
+    with codes near -128, so that rq - D*zq comes close to +-255*D (65 280 at head_dim 256, where it no longer splits into
+    two 7-bit digits) and the code row sums reach +-127*D.  The integer zero-point correction of the score kernels
+    has to stay exact for every pairing of such query and key rows, forward and backward."""
+    B, H, N = 1, 2, 192
+    g = torch.Generator().manual_seed(D)
+    def rows():
+        x = torch.randn((B, H, N, D), generator=g) * 0.05
+        hi = 0.08 * (0.97 + 0.03 * torch.rand((B, H, N, D), generator=g))
+        hi[..., 0] = 0.0
+        x[:, :, 0::3] = hi[:, :, 0::3]          # all positive, minimum 0: zero point -128, codes near +127
+        x[:, :, 1::3] = -hi[:, :, 1::3]         # all negative, maximum 0: zero point +127, codes near -128
+        return x.to(torch.bfloat16)
+    q, k = rows(), rows().flip(2)
+    v = torch.randn((B, H, N, D), generator=g).to(torch.bfloat16)
+    do = torch.randn((B, H, N, D), generator=g).to(torch.bfloat16)
+    sm = 1.0 / math.sqrt(D)
+    for causal in (False, True):
+        qq, kq, o, lse, dq, dk, dv = _fwd_bwd(qfa, q, k, v, do, causal, sm)
+        c = qq.rowsum.cpu().long().reshape(B, H, N) - D * qq.zero_point.cpu().long().reshape(B, H, N)
+        assert c.max() > 240 * D and c.min() < -240 * D, "the inputs do not reach the range they are meant to test"
+        assert kq.rowsum.abs().max() > 120 * D
+        qh = oracle.dequantize_per_token(qq.codes.cpu(), qq.scale.cpu(), qq.zero_point.cpu(), torch.float64)
+        kh = oracle.dequantize_per_token(kq.codes.cpu(), kq.scale.cpu(), kq.zero_point.cpu(), torch.float64)
+        o_ref, lse_ref = oracle.attn_fwd(qh, kh, v, causal, sm)
+        assert_close(f"O causal={causal}", o.cpu(), o_ref)
+        assert max_abs(lse.cpu(), lse_ref) < 2.0 ** -8
+        want, spreads = _oracle_bwd(qq, kq, v, do, o, causal, sm)
+        _check_grads(f" causal={causal}", (dq.cpu(), dk.cpu(), dv.cpu()), want, spreads)
+
+
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_delta_kernel(qfa, D):
     from quant_flash_attn_amd import _lib
-    o = torch.randn(2, 3, 130, 128, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
-    do = torch.randn(2, 3, 130, 128, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16)
+    o = torch.randn(2, 3, 130, D, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    do = torch.randn(2, 3, 130, D, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16)
     og, dog = o.to(DEV), do.to(DEV)
     delta = torch.empty(2, 3, 130, dtype=torch.float32, device=DEV)
     s = (og.stride(0), og.stride(1), og.stride(2))
-    rc = _lib.lib().qfa_bwd_delta(og.data_ptr(), dog.data_ptr(), delta.data_ptr(), _lib.QFA_BF16, 2, 3, 130, 128,
+    rc = _lib.lib().qfa_bwd_delta(og.data_ptr(), dog.data_ptr(), delta.data_ptr(), _lib.QFA_BF16, 2, 3, 130, D,
                                   *s, *s, torch.cuda.current_stream().cuda_stream)
     _lib.check(rc, "qfa_bwd_delta")
     assert max_abs(delta.cpu(), oracle.bwd_delta(o, do)) < 1e-4
@@ -117,9 +151,10 @@ def test_full_size_sampled_heads_and_properties(qfa, config, B, H, N, D, causal)
     assert (lhs - rhs).abs().max() < 0.02 * math.sqrt(N)
 
 
-def test_autograd_entry_points(qfa):
+@pytest.mark.parametrize("D", [128, 256])
+def test_autograd_entry_points(qfa, D):
     """quant_flash_attn_qkv(q,k,v,causal,sm) and the reference-style quant_flash_attn(q, kv, kv_quant, sm)."""
-    B, H, N, D = 2, 2, 256, 128
+    B, H, N = 2, 2, 256
     q, k, v, do = make_inputs("offset", B, H, N, D, seed=21)
     sm = 1.0 / math.sqrt(D)
     qg, kg, vg = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
@@ -136,7 +171,9 @@ def test_autograd_entry_points(qfa):
 
 @pytest.mark.parametrize("Z,H,Nq,Nkv,D", [(2, 4, 18, 512, 64), (2, 8, 32, 1024, 128), (4, 16, 16, 2048, 64), (1, 2, 17, 1023, 128),
                                           (3, 5, 97, 689, 128),      # the reference's shapes (test_accuracy.py:35-45, small batch)
-                                          (1, 2, 600, 700, 128)])    # query block past the shared-KV kernels: INT8-score path
+                                          (1, 2, 600, 700, 128),     # query block past the shared-KV kernels: INT8-score path
+                                          (2, 2, 97, 689, 256),      # compute_flops.py:94 sweeps head_dim 256
+                                          (1, 2, 1100, 1200, 256)])  # past the shared-KV kernels at head_dim 256
 def test_reference_entry_point_shared_kv(qfa, Z, H, Nq, Nkv, D):
     """The reference's own test (test_accuracy.py:47-133): fp16 q, kv ~ N(0,1), seed 20, quantize kv
     externally, forward + backward, against un-quantized fp16-input attention at its tolerances
@@ -160,10 +197,10 @@ def test_reference_entry_point_shared_kv(qfa, Z, H, Nq, Nkv, D):
     assert torch.allclose(kvg.grad.cpu().double(), kvr.grad, atol=1e-2, rtol=2e-2)
     # shared-KV oracle on the same codes: Q as it is for the shared-KV kernels (the reference's
     # computation), quantized per token where the INT8-score kernels take over
-    from quant_flash_attn_amd.quant_flash_attn import SHARED_KV_MAX_Q
+    from quant_flash_attn_amd.quant_flash_attn import shared_kv_max_q
     codes, scale, zp = (t.cpu() for t in kv_quant)
     qh = q
-    if Nq > SHARED_KV_MAX_Q:
+    if Nq > shared_kv_max_q(D):
         qc, _, zq, sq, _ = oracle.quantize_per_token(q)
         qh = oracle.dequantize_per_token(qc, sq, zq, torch.float64)
     o_ref, _ = oracle.legacy_fwd(qh, codes, scale, zp, sm)

@@ -32,10 +32,10 @@ def _scores(kind, q, k, Nk, g):
     return q, k
 
 
-def test_forward_random_sweep(qfa):
-    rng = random.Random(1234)
-    for it in range(96):
-        D = rng.choice((64, 128))
+def _forward_sweep(qfa, seed, dims, iters):
+    rng = random.Random(seed)
+    for it in range(iters):
+        D = rng.choice(dims)
         dt = rng.choice((torch.bfloat16, torch.float16))
         causal = rng.random() < 0.5
         B, H = rng.choice(((1, 1), (1, 2), (2, 2)))
@@ -56,6 +56,14 @@ def test_forward_random_sweep(qfa):
         case = f"case {it}: {kind} B{B} H{H} Nq{Nq} Nk{Nk} D{D} {dt} causal={causal}"
         assert_close(case + " O", o.cpu(), o_ref)
         assert max_abs(lse.cpu(), lse_ref) < 2.0 ** -8 * max(1.0, float(lse_ref.abs().max()) / 64), case
+
+
+def test_forward_random_sweep(qfa):
+    _forward_sweep(qfa, 1234, (64, 128), 96)
+
+
+def test_forward_random_sweep_head_dim_256(qfa):
+    _forward_sweep(qfa, 2560, (256,), 40)
 
 
 def test_shared_kv_random_sweep(qfa):
@@ -93,12 +101,10 @@ def test_shared_kv_random_sweep(qfa):
         assert torch.isfinite(dq).all() and torch.isfinite(dkv).all(), case
 
 
-def test_backward_random_sweep(qfa):
-    """Forward + backward of the INT8-score kernels; head counts from 1 to 20 so that the causal dispatch
-    groups (2 to 8 heads) come out full, partial and absent."""
-    rng = random.Random(777)
-    for it in range(72):
-        D = rng.choice((64, 128))
+def _backward_sweep(qfa, seed, dims, iters):
+    rng = random.Random(seed)
+    for it in range(iters):
+        D = rng.choice(dims)
         dt = rng.choice((torch.bfloat16, torch.float16))
         causal = rng.random() < 0.6
         B, H = rng.choice(((1, 1), (1, 2), (2, 2), (3, 3), (2, 5), (1, 16), (4, 5)))
@@ -128,3 +134,13 @@ def test_backward_random_sweep(qfa):
         assert_close(case + " dK", dk.cpu(), rk, scaled=True, spread=nk)
         assert_close(case + " dV", dv.cpu(), rv, scaled=True, spread=nv)
         assert torch.isfinite(dq).all() and torch.isfinite(dk).all() and torch.isfinite(dv).all(), case
+
+
+def test_backward_random_sweep(qfa):
+    """Forward + backward of the INT8-score kernels; head counts from 1 to 20 so that the causal dispatch
+    groups (2 to 8 heads) come out full, partial and absent."""
+    _backward_sweep(qfa, 777, (64, 128), 72)
+
+
+def test_backward_random_sweep_head_dim_256(qfa):
+    _backward_sweep(qfa, 2561, (256,), 32)
