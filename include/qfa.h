@@ -37,7 +37,7 @@ extern "C" {
 
 /* argument errors */
 #define QFA_EINVAL (-1)       /* null pointer, non-positive size, bad dtype code, misaligned pointer/stride */
-#define QFA_EUNSUPPORTED (-2) /* well-formed but not implemented (head_dim, causal with Nq != Nk, ...) */
+#define QFA_EUNSUPPORTED (-2) /* well-formed but not implemented (head_dim, causal with Nq > Nk, ...) */
 
 int qfa_version(void);
 const char *qfa_last_error(void);
@@ -88,7 +88,9 @@ int qfa_dequant_per_token(const int8_t *codes, const void *scale, int scale_dtyp
  *   qc,kc  int8 [B,H,Nq|Nk,D];  sq,sk float, zq,zk int8, rq,rk int32: dense [B*H*Nq|Nk]
  *   v, o   [B,H,Nk|Nq,D] of io_dtype (QFA_BF16 or QFA_F16);  lse float [B*H*Nq]
  *   D in {64, 128, 256} (the widths compute_flops.py:94 sweeps; also for qfa_attn_bwd and qfa_bwd_delta).
- *   causal != 0 requires Nq == Nk.  All tensors 16-byte aligned, strides
+ *   causal != 0: query i keeps the keys j <= i + (Nk - Nq), the mask aligned to the last key, which needs
+ *   Nq <= Nk (with Nq == Nk the rule row >= col of flash_attn_triton.py:50; the reference has no other case:
+ *   a block of queries at the end of a longer key sequence).  All tensors 16-byte aligned, strides
  *   multiples of 16 bytes, token strides below 2^23 elements, Nq and Nk at most 2^28
  *   (QFA_EUNSUPPORTED otherwise).
  */

@@ -155,10 +155,12 @@ def int_scores(qc: torch.Tensor, zq: torch.Tensor, kc: torch.Tensor, zk: torch.T
 
 # --------------------------------------------------------------------------- attention
 def _causal_mask(nq: int, nk: int, device=None) -> torch.Tensor:
-    """True where the score is kept: row >= col (flash_attn_triton.py:50)."""
+    """True where the score is kept: row >= col (flash_attn_triton.py:50).  The reference only has nq == nk; for
+    nq < nk the mask is aligned to the last key (row + nk - nq >= col), so that the rows are the last nq rows of the
+    square case -- what a chunk of queries at the end of a longer key sequence needs."""
     i = torch.arange(nq, device=device)[:, None]
     j = torch.arange(nk, device=device)[None, :]
-    return i >= j
+    return i + (nk - nq) >= j
 
 
 def attn_fwd(qh: torch.Tensor, kh: torch.Tensor, v: torch.Tensor, causal: bool, sm_scale: float,

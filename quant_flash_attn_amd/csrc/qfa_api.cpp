@@ -97,7 +97,8 @@ static int check_attn_common(const char *who, const AttnArgs &a) {
     return set_error(QFA_EUNSUPPORTED, "%s: head_dim %d not in {64, 128, 256}", who, a.D);
   if (!(a.sm_scale > 0.0f) || !(a.sm_scale < 3.0e38f))
     return set_error(QFA_EINVAL, "%s: sm_scale must be a positive finite number", who);
-  if (a.causal && a.Nq != a.Nk) return set_error(QFA_EUNSUPPORTED, "%s: causal needs Nq == Nk", who);
+  if (a.causal && a.Nq > a.Nk)
+    return set_error(QFA_EUNSUPPORTED, "%s: causal needs Nq <= Nk (the mask is aligned to the last key)", who);
   if (!aligned16(a.qc) || !aligned16(a.kc) || !aligned16(a.v) || !aligned16(a.o))
     return set_error(QFA_EINVAL, "%s: qc, kc, v, o must be 16-byte aligned", who);
   if (!strides_ok(a.sqb, a.sqh, a.sqn, a.D, 1) || !strides_ok(a.skb, a.skh, a.skn, a.D, 1) ||

@@ -324,7 +324,8 @@ __global__ __launch_bounds__(DqShape<D>::THREADS, DqShape<D>::WAVES_PER_SIMD) vo
   const int q_first = m0 + wave * 32, q_last = q_first + 31;
 
   int kv_end = a.Nk;
-  if (CAUSAL) kv_end = min(a.Nk, m0 + DQ_BLK);
+  const int coff = CAUSAL ? a.Nk - a.Nq : 0;   // causal: query i keeps keys j <= i + coff (mask aligned to the last key)
+  if (CAUSAL) kv_end = min(a.Nk, m0 + DQ_BLK + coff);
   const int ntiles = (kv_end + BWD_TILE - 1) / BWD_TILE;
 
   // full tiles: per-thread offsets computed once, one copy instruction per chunk afterwards
@@ -403,7 +404,7 @@ __global__ __launch_bounds__(DqShape<D>::THREADS, DqShape<D>::WAVES_PER_SIMD) vo
         float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, f[v] * sk4[bb], nlse2));
         if (MASKED) {
           const int j = j0 + jl + bb;
-          if ((CAUSAL && j > qi) || j >= a.Nk) p = 0.f;
+          if ((CAUSAL && j > qi + coff) || j >= a.Nk) p = 0.f;
         }
         ds[v] = p * dp[v];
       }
@@ -433,8 +434,8 @@ __global__ __launch_bounds__(DqShape<D>::THREADS, DqShape<D>::WAVES_PER_SIMD) vo
         if (nb == NBLK - 1) load_tile_b(t + 1);
       }
       const int jb = j0 + 32 * nb;
-      if ((jb >= a.Nk) || (CAUSAL && jb > q_last)) continue;               // wave-uniform
-      if ((CAUSAL && jb + 31 > q_first) || (jb + 32 > a.Nk)) block(t, nb, std::true_type{});
+      if ((jb >= a.Nk) || (CAUSAL && jb > q_last + coff)) continue;        // wave-uniform
+      if ((CAUSAL && jb + 31 > q_first + coff) || (jb + 32 > a.Nk)) block(t, nb, std::true_type{});
       else block(t, nb, std::false_type{});
     }
     dma_wait();
@@ -548,7 +549,8 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
   const float sk_j = __builtin_bit_cast(float, ck[2 * BWD_TILE + kl]);
   const int k_first = n0 + pair * 32, k_last = k_first + 31;
 
-  const int it0 = CAUSAL ? n0 / BWD_TILE : 0;
+  const int coff = CAUSAL ? a.Nk - a.Nq : 0;   // causal: key j is seen by the queries i >= j - coff
+  const int it0 = CAUSAL ? max(n0 - coff, 0) / BWD_TILE : 0;
   const int ntiles = a.tiles_q;
 
   // full tiles: per-thread offsets computed once, one copy instruction per chunk afterwards
@@ -640,7 +642,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
         float p = __builtin_amdgcn_exp2f(__builtin_fmaf(a4[aa][bb], f[4 * aa + bb] * sk_j, nl4[aa][bb]));
         if (MASKED) {
           const int i = i0 + il + bb;
-          if ((CAUSAL && kj > i) || i >= a.Nq || kj >= a.Nk) p = 0.f;
+          if ((CAUSAL && kj > i + coff) || i >= a.Nq || kj >= a.Nk) p = 0.f;
         }
         pp[4 * aa + bb] = p;
       }
@@ -721,8 +723,8 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, DkvShape<D>::WAVES_PER_SIMD) 
   // The two roles run separate loops with the same barrier sequence (one per 32-query block).
   auto block_flags = [&](int t, int mbk, bool &on, bool &masked) {
     const int ib = t * BWD_TILE + 32 * mbk;
-    on = (ib < a.Nq) && (!CAUSAL || ib + 31 >= k_first);                               // wave-uniform
-    masked = (CAUSAL && ib < k_last) || (ib + 32 > a.Nq) || (k_last >= a.Nk);
+    on = (ib < a.Nq) && (!CAUSAL || ib + 31 + coff >= k_first);                        // wave-uniform
+    masked = (CAUSAL && ib + coff < k_last) || (ib + 32 > a.Nq) || (k_last >= a.Nk);
   };
   // Block (t, mbk): first phase | barrier | second phase; all reads of the tile buffers happen in first phases.
   // 64-query tiles (two blocks): the next tile's copy goes out in two halves around the barrier of the tile's first

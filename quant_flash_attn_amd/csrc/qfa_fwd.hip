@@ -121,7 +121,10 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
 
   // ---- tile range
   int kv_end = a.Nk;
-  if (CAUSAL) kv_end = min(a.Nk, m0 + FWD_BM);
+  // causal: query i keeps keys j <= i + coff, the mask aligned to the last key (coff = Nk - Nq >= 0; the rule
+  // row >= col when Nq == Nk)
+  const int coff = CAUSAL ? a.Nk - a.Nq : 0;
+  if (CAUSAL) kv_end = min(a.Nk, m0 + FWD_BM + coff);
   const int ntiles = (kv_end + FWD_BN - 1) / FWD_BN;
 
   // ---- tile copies: K and V by direct loads, the per-key constants through registers
@@ -229,7 +232,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
         float uu = f[4 * aa + bb] * sk4[bb];
         if (MASKED) {
           const int j = j0 + jl + bb;
-          if ((CAUSAL && j > qi) || j >= a.Nk) uu = -INFINITY;
+          if ((CAUSAL && j > qi + coff) || j >= a.Nk) uu = -INFINITY;
         }
         u[4 * aa + bb] = uu;
         mt = fmaxf(mt, uu);
@@ -306,7 +309,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
 
   // tiles [0, t_hot) contain no masked score for this wave (wave-uniform)
   int t_hot = a.Nk / FWD_BN;
-  if (CAUSAL) t_hot = min(t_hot, (q_first + 1) / FWD_BN);
+  if (CAUSAL) t_hot = min(t_hot, (q_first + coff + 1) / FWD_BN);
   t_hot = min(t_hot, ntiles);
 
   int kb_cur = 0, kb_nxt = 1, kb_free = 2;   // K/constant buffers of tile t, t+1, and the one to refill
@@ -511,7 +514,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
       const int jb = j0 + 32 * nb;
-      if ((CAUSAL && jb > q_last) || jb >= a.Nk) continue;   // wave-uniform: nothing to keep
+      if ((CAUSAL && jb > q_last + coff) || jb >= a.Nk) continue;   // wave-uniform: nothing to keep
       i32x16 s;
       float u[16];
       qk_block(kb_cur, nb, s);

@@ -225,7 +225,8 @@ class QuantFlashAttnQKV(torch.autograd.Function):
     """forward(ctx, q, k, v, causal, sm_scale) -> o   (argument order of flash_attn_triton.py:441).
 
     q, k, v: [B,H,N,D] bf16 / fp16 (fp32 is accepted: V and O then pass through bf16).
-    causal keeps key j for query i when j <= i (flash_attn_triton.py:50)."""
+    causal keeps key j for query i when j <= i (flash_attn_triton.py:50); with fewer queries than keys the mask is
+    aligned to the last key (j <= i + Nk - Nq)."""
 
     @staticmethod
     def forward(ctx, q, k, v, causal, sm_scale):

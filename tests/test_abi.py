@@ -50,7 +50,7 @@ def test_argument_errors_need_no_gpu(qfa):
     def fwd(Nq=128, Nk=128, D=64, sm=0.125, causal=0, io=2):
         s = (Nq * D * 2, Nq * D, D)
         return L.qfa_attn_fwd(*([ok_ptr] * 11), io, 1, 2, Nq, Nk, D, *s, *s, *s, *s, sm, causal, None)
-    assert fwd(Nq=64, Nk=128, causal=1) == -2 and b"causal" in L.qfa_last_error()
+    assert fwd(Nq=192, Nk=128, causal=1) == -2 and b"causal" in L.qfa_last_error()   # more queries than keys
     assert fwd(sm=0.0) == -1 and b"sm_scale" in L.qfa_last_error()
     assert fwd(D=96) == -2 and b"head_dim" in L.qfa_last_error()
     assert fwd(io=0) == -1 and b"io_dtype" in L.qfa_last_error()

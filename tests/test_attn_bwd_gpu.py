@@ -62,6 +62,12 @@ CASES = [
     (1, 2, 333, 333, 256, True, "uniform", torch.bfloat16),     # ragged, causal
     (2, 2, 97, 689, 256, False, "offset", torch.float16),       # short Q, long ragged KV
     (1, 3, 200, 200, 256, False, "uniform", torch.bfloat16),    # ragged
+    # causal with fewer queries than keys: the mask is aligned to the last key
+    (2, 2, 128, 384, 128, True, "normal", torch.bfloat16),
+    (1, 3, 97, 689, 128, True, "offset", torch.float16),        # ragged both ways, offset 592
+    (1, 2, 200, 333, 64, True, "uniform", torch.bfloat16),
+    (1, 2, 1, 300, 128, True, "normal", torch.bfloat16),        # one query: sees every key
+    (2, 2, 160, 200, 256, True, "offset", torch.bfloat16),
 ]
 
 

@@ -46,6 +46,20 @@ def test_fwd_special_cases():
     q, k = _rand(1, 1, 9, 4, seed=5), _rand(1, 1, 9, 4, seed=6)
     o, _ = oracle.attn_fwd(q, k, v, True, 0.5)
     assert torch.allclose(o[..., 0, :], v[..., 0, :])
+    # causal with fewer queries than keys: the rows are the last rows of the square case; and against the library
+    # mask built independently (tril with a diagonal offset)
+    q9, k9 = _rand(1, 1, 9, 4, seed=5), _rand(1, 1, 9, 4, seed=6)
+    o_sq, lse_sq = oracle.attn_fwd(q9, k9, v, True, 0.5)
+    o_r, lse_r = oracle.attn_fwd(q9[..., 5:, :], k9, v, True, 0.5)
+    assert torch.allclose(o_r, o_sq[..., 5:, :]) and torch.allclose(lse_r, lse_sq[..., 5:])
+    keep = torch.ones(4, 9, dtype=torch.bool).tril(diagonal=5)
+    ref = F.scaled_dot_product_attention(q9[..., 5:, :], k9, v, attn_mask=keep, scale=0.5)
+    assert torch.allclose(o_r, ref)
+    dq_r, dk_r, dv_r = oracle.attn_bwd(q9[..., 5:, :], k9, v, torch.ones(1, 1, 4, 4, dtype=torch.float64), True, 0.5)
+    g = torch.zeros(1, 1, 9, 4, dtype=torch.float64)
+    g[..., 5:, :] = 1.0
+    dq_s, dk_s, dv_s = oracle.attn_bwd(q9, k9, v, g, True, 0.5)
+    assert torch.allclose(dq_r, dq_s[..., 5:, :]) and torch.allclose(dk_r, dk_s) and torch.allclose(dv_r, dv_s)
     # Nq != Nk, non causal: shapes and a one-key limit
     o, lse = oracle.attn_fwd(q[..., :3, :], k[..., :1, :], v[..., :1, :], False, 0.5)
     assert torch.allclose(o, v[..., :1, :].expand(1, 1, 3, 4))
