@@ -257,6 +257,48 @@ class QuantFlashAttnQKV(torch.autograd.Function):
 quant_flash_attn_qkv = QuantFlashAttnQKV.apply
 
 
+class QuantFlashAttnQuantizedKV(torch.autograd.Function):
+    """forward(ctx, q, k_fp16, v_fp16, k_quant, v_quant, causal, sm_scale) -> o; backward -> (dq, dk, dv, None...).
+
+    The reference's contract (quant_flash_attn.py:178-237: the keys and values arrive as INT8 codes with per-token
+    scale and zero point, a 16-bit placeholder leaf receives the gradient) with K and V as two separately quantized
+    tensors instead of one shared tensor, and a causal flag.  k_quant and v_quant are (codes, scale, zero_point)
+    tuples as asymmetric_quant_per_token returns them; k_fp16 and v_fp16 are only placeholders.
+    The K codes are used as they are (INT8 scores); V is dequantized once per call by the HIP dequantizer into a
+    16-bit tensor that the P.V product streams: converting int8 V inside the attention kernel would add about 110
+    vector instructions per 32x32 block to a loop that is bound by its vector instructions, the separate pass adds
+    a read of the codes and one 16-bit write and read (8 % of the forward at B4 H32 N4096 D128)."""
+
+    @staticmethod
+    def forward(ctx, q, k_fp16, v_fp16, k_quant, v_quant, causal, sm_scale):
+        kc, ks, kz = k_quant
+        vc, vs, vz = v_quant
+        _lib.require_gpu(q, kc, ks, kz, vc, vs, vz)
+        if q.dim() != 4 or kc.dim() != 4 or kc.shape != vc.shape or q.shape[-1] != kc.shape[-1] or q.shape[:2] != kc.shape[:2]:
+            raise ValueError(f"shape mismatch: q {tuple(q.shape)}, k codes {tuple(kc.shape)}, v codes {tuple(vc.shape)}")
+        io = _io_dtype(q)
+        qq = quantize_for_attention(q)
+        kq = QuantizedTokens(kc, ks.to(torch.float32), kz, kc.sum(dim=-1, keepdim=True, dtype=torch.int32))
+        v16 = dequantize_per_token(vc, vs, vz, io)
+        o, lse = attn_fwd_quantized(qq, kq, v16, causal, sm_scale)
+        ctx.save_for_backward(*qq, *kq, v16, o, lse)
+        ctx.causal, ctx.sm_scale = bool(causal), float(sm_scale)
+        ctx.in_dtypes = (q.dtype, k_fp16.dtype, v_fp16.dtype)
+        return o.to(q.dtype)
+
+    @staticmethod
+    def backward(ctx, do):
+        t = ctx.saved_tensors
+        qq, kq = QuantizedTokens(*t[0:4]), QuantizedTokens(*t[4:8])
+        v16, o, lse = t[8], t[9], t[10]
+        dq, dk, dv = attn_bwd_quantized(qq, kq, v16, o, do.to(v16.dtype), lse, ctx.causal, ctx.sm_scale)
+        dq_t, dk_t, dv_t = ctx.in_dtypes
+        return dq.to(dq_t), dk.to(dk_t), dv.to(dv_t), None, None, None, None
+
+
+quant_flash_attn_quantized_kv = QuantFlashAttnQuantizedKV.apply
+
+
 class QuantFlashAttention(torch.autograd.Function):
     """forward(ctx, q, kv_fp16, kv_quant, sm_scale) -> o; backward -> (dq, dkv, None, None).
 

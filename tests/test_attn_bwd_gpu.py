@@ -175,6 +175,32 @@ def test_autograd_entry_points(qfa, D):
     _check_grads("", (qg.grad.cpu(), kg.grad.cpu(), vg.grad.cpu()), want, spreads)
 
 
+@pytest.mark.parametrize("B,H,Nq,Nk,D,causal", [(2, 2, 256, 256, 128, True), (1, 3, 100, 333, 64, False),
+                                                (1, 2, 128, 320, 256, True)])
+def test_quantized_kv_entry_point(qfa, B, H, Nq, Nk, D, causal):
+    """K and V as two INT8 tensors (codes, fp16 scale, zero point, as asymmetric_quant_per_token returns them):
+    O and the gradients against the oracle on the dequantized operands, the gradients of K and V landing in the
+    16-bit placeholder leaves as in the reference's contract (quant_flash_attn.py:232-237)."""
+    N = max(Nq, Nk)
+    q, k, v, do = make_inputs("offset", B, H, N, D, seed=77 + D, dtype=torch.float16)
+    q, do = q[:, :, :Nq].contiguous(), do[:, :, :Nq].contiguous()
+    k, v = k[:, :, :Nk].contiguous(), v[:, :, :Nk].contiguous()
+    sm = 1.0 / math.sqrt(D)
+    qg, kg, vg = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    k_quant = qfa.asymmetric_quant_per_token(kg.detach())
+    v_quant = qfa.asymmetric_quant_per_token(vg.detach())
+    o = qfa.quant_flash_attn_quantized_kv(qg, kg, vg, k_quant, v_quant, causal, sm)
+    o.backward(do.to(DEV))
+    qc, _, zq, sq, _ = oracle.quantize_per_token(q)
+    qh = oracle.dequantize_per_token(qc, sq, zq, torch.float64)
+    kh = oracle.dequantize_per_token(*(t.cpu() for t in k_quant), torch.float64)       # fp16 scale, as stored
+    vh = oracle.dequantize_per_token(*(t.cpu() for t in v_quant)).to(torch.float16)    # what the P.V product streams
+    o_ref, _ = oracle.attn_fwd(qh, kh, vh, causal, sm)
+    want, spreads = oracle.attn_bwd(qh, kh, vh, do, causal, sm, o=o.detach().cpu(), spread=True)
+    assert_close("O", o.detach().cpu(), o_ref)
+    _check_grads("", (qg.grad.cpu(), kg.grad.cpu(), vg.grad.cpu()), want, spreads)
+
+
 @pytest.mark.parametrize("Z,H,Nq,Nkv,D", [(2, 4, 18, 512, 64), (2, 8, 32, 1024, 128), (4, 16, 16, 2048, 64), (1, 2, 17, 1023, 128),
                                           (3, 5, 97, 689, 128),      # the reference's shapes (test_accuracy.py:35-45, small batch)
                                           (1, 2, 600, 700, 128),     # query block past the shared-KV kernels: INT8-score path
