@@ -42,10 +42,10 @@ PEAK_INT8_TOPS = 5000.0
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per forward launch at the headline configuration, measured with rocprofv3 --pmc:
-# FETCH_SIZE 195 063 KiB x 2.000 (calibration: 256 MiB copy reads 131 085) + WRITE_SIZE 133 195 KiB x 1.000
+# FETCH_SIZE 197 055 KiB x 2.000 (calibration: 256 MiB copy reads 131 086) + WRITE_SIZE 133 120 KiB x 1.000
 # (profiles/kernels_B4_H32_N4096_D128_causal_bf16.md); algorithmic bytes are 395 MiB -- the causal dispatch
 # order keeps four heads in flight per XCD, more than its L2 holds, and the re-reads show up here
-FWD_TRAFFIC_BYTES = (193050 * 2 + 133233) * 1024
+FWD_TRAFFIC_BYTES = (197055 * 2 + 133120) * 1024
 
 
 def flops_fwd(B, H, Nq, Nk, D, causal):
@@ -258,7 +258,9 @@ def main():
 
     if not args.quick:
         others = {"long_context_B1_H16_N16384_D128_noncausal": (1, 16, 16384, 128, False, "outlier"),
-                  "small_head_B16_H16_N2048_D64_causal": (16, 16, 2048, 64, True, "uniform")}
+                  "small_head_B16_H16_N2048_D64_causal": (16, 16, 2048, 64, True, "uniform"),
+                  # the widest head compute_flops.py:94 sweeps, at the headline's token count and model width
+                  "wide_head_B4_H16_N4096_D256_causal": (4, 16, 4096, 256, True, "offset")}
         del q, k, v, do, qq, kq, o, lse
         for name, (b2, h2, n2, d2, c2, dist) in others.items():
             q2, k2, v2, do2 = (t.to(dev) for t in make_inputs(dist, b2, h2, n2, d2, seed=0))
