@@ -105,6 +105,40 @@ def test_scores_jump_far_above_the_running_reference(qfa, D, dtype, jump, causal
     assert max_abs(lse.cpu(), lse_ref) < LSE_TOL * max(1.0, float(lse_ref.abs().max()) / 64)
 
 
+@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("causal", [False, True])
+def test_constant_rows_at_the_clamps_give_exact_integer_scores(qfa, D, causal):
+    """Constant rows of +-300 quantize to scale 1, codes +127 / -128 and zero points -128 / +127: the largest integer
+    score, code row sums and zero-point terms the kernels can meet (+-255 * 255 * D), all of one sign at once.  With
+    sm_scale = 4 every query of such a row gives equal weight to the keys of its own sign and none to the others,
+    and an integer score off by one would give one key e^4 times the weight of its peers: O must be the mean of V
+    over those keys.  Checks the exactness of the INT8 product plus the zero-point correction at the end of its
+    range, in the pipelined loop (first tile) and in the masked one (ragged second tile)."""
+    B, H, Nq, Nk = 1, 2, 96, 96
+    g = torch.Generator().manual_seed(3 * D + causal)
+    def rows(n):
+        x = torch.randn((B, H, n, D), generator=g)
+        x[:, :, 0::3] = 300.0
+        x[:, :, 1::3] = -300.0
+        return x.to(torch.bfloat16)
+    q, k = rows(Nq), rows(Nk)
+    v = torch.randn((B, H, Nk, D), generator=g).to(torch.bfloat16)
+    sm = 4.0
+    qq, kq, o, lse = _run(qfa, q, k, v, causal, sm)
+    assert qq.codes[0, 0, 0].eq(127).all() and qq.zero_point[0, 0, 0].item() == -128 and qq.scale[0, 0, 0].item() == 1.0
+    assert kq.codes[0, 0, 1].eq(-128).all() and kq.zero_point[0, 0, 1].item() == 127
+    o_ref, lse_ref = _oracle_fwd(qq, kq, v, causal, sm)
+    rows_pm = [i for i in range(Nq) if i % 3 != 2 and not (causal and i < 3)]
+    assert_close("O of the constant rows", o.cpu()[:, :, rows_pm], o_ref[:, :, rows_pm])
+    # and directly: the mean of V over the visible keys of the query's sign
+    vd = v.double()
+    for i in rows_pm[:8] + rows_pm[-8:]:
+        keys = [j for j in range(Nk) if j % 3 == i % 3 and (not causal or j <= i)]
+        assert max_abs(o.cpu()[:, :, i], vd[:, :, keys].mean(2)) < 2e-2, (i, len(keys))
+    rel = ((lse.cpu().double() - lse_ref).abs() / lse_ref.abs().clamp_min(1.0))[:, :, rows_pm]
+    assert float(rel.max()) < 1e-6
+
+
 def test_fp32_plumbing_configuration(qfa):
     """B1 H4 N256 D64 fp32 q,k,v, seed 0, non-causal, through the autograd entry point."""
     torch.manual_seed(0)
