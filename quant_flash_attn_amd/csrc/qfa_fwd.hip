@@ -117,24 +117,6 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
     const int hi = c >> SH, lo = c & ((1 << SH) - 1);
     corr_q[0] = g == 0 ? pack2<T>((float)(-zq_i), (float)(-zq_i)) : pack2<T>((float)(-(hi * (1 << SH))), (float)(-lo));
   }
-  // head_dim 64: the int32 accumulators of the score product start from the bit pattern of the float 9 * 2^20
-  // (= 2^23 + 2^20) instead of zero.  With |S| <= 2^20 the integer 0x4B100000 + S, read as a float, IS
-  // 9 * 2^20 + S (all of [2^23, 2^23 + 2^21] lies in the binade whose spacing is 1), so the accumulator needs no
-  // conversion: sixteen vector instructions less per 32x32 block, 6 % of this kernel.  The constant leaves again in
-  // the correction MFMA as a fifth term 1024 * (-9216), both factors exact in either 16-bit type.  Exact in any
-  // order of accumulation: the constant, the scores and all four zero-point terms together stay below
-  // 10 485 760 + 1 040 384 + 2 072 640 + 32 258 < 2^24.  At head_dim 128 the same sum could pass 2^24 before the
-  // constant is taken out (and the loop there gains nothing: measured), so wider heads convert.
-  constexpr bool BIASED = D <= 64;
-  u32x4 corr_k_const = {0u, 0u, 0u, 0u};   // slots of the key-side operand that do not depend on the key
-  i32x16 s_init;
-#pragma unroll
-  for (int v = 0; v < 16; ++v) s_init[v] = BIASED ? 0x4B100000 : 0;
-  if (BIASED) {
-    corr_q[1] = g == 0 ? pack2<T>(-9216.0f, 0.0f) : 0u;
-    corr_k_const[1] = g == 0 ? pack2<T>(1024.0f, 0.0f) : 0u;
-    asm volatile("" : "+v"(s_init));   // sixteen registers for the whole kernel, not sixteen moves per block
-  }
   const int q_first = m0 + wave * 32, q_last = q_first + 31;
 
   // ---- tile range
@@ -208,12 +190,8 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   // S^T block nb (32 keys) of the tile held in K buffer `buf`, for this wave's 32 queries
   auto qk_block = [&](int buf, int nb, i32x16 &s) {
     const unsigned char *ks_ = smem + SM::OFF_K + buf * SM::K_BYTES;
-    if constexpr (BIASED) {
-      s = s_init;
-    } else {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) s[v] = 0;
-    }
+    for (int v = 0; v < 16; ++v) s[v] = 0;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const i32x4 kf =
@@ -240,13 +218,9 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
     const float *skp = reinterpret_cast<const float *>(cb);
     const unsigned *dgp = reinterpret_cast<const unsigned *>(cb + FWD_BN * 4);
     f32x16 f;
-    if constexpr (BIASED) {
-      f = __builtin_bit_cast(f32x16, s);
-    } else {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
-    }
-    u32x4 corr_k = {dgp[2 * (32 * nb + lr) + g], corr_k_const[1], 0u, 0u};
+    for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
+    u32x4 corr_k = {dgp[2 * (32 * nb + lr) + g], 0u, 0u, 0u};
     f = mfma_16b<T>(corr_k, corr_q, f);
     float mt = -INFINITY;
 #pragma unroll
@@ -416,12 +390,8 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(1);
       // INT8 product of block b+1 under the exponentials of the first 16 keys of block b
-      if constexpr (BIASED) {
-        s = s_init;
-      } else {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) s[v] = 0;
-      }
+      for (int v = 0; v < 16; ++v) s[v] = 0;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) s = mfma_i8(kf[ks], qf[ks], s);
       float l0, l1;
@@ -439,7 +409,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa)
         sk4[aa] = *reinterpret_cast<const f32x4 *>(cb + (32 * cnb + 8 * aa + 4 * g) * 4);
-      const u32x4 corr_k = {reinterpret_cast<const unsigned *>(cb + FWD_BN * 4)[2 * (32 * cnb + lr) + g], corr_k_const[1], 0u, 0u};
+      const u32x4 corr_k = {reinterpret_cast<const unsigned *>(cb + FWD_BN * 4)[2 * (32 * cnb + lr) + g], 0u, 0u, 0u};
       __builtin_amdgcn_sched_barrier(0);
       // P.V of the first 16 keys under the exponentials of the second 16 and the conversion of the next
       // block's raw scores; their zero-point correction (one MFMA) goes last, so that its result has the
@@ -458,12 +428,8 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
         for (int v = 0; v < 16; ++v) sm = fmaxf(sm, u[v]);
         l_run = fmaxf(l_run, sm);
       }
-      if constexpr (BIASED) {
-        f = __builtin_bit_cast(f32x16, s);
-      } else {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
-      }
+      for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
       __builtin_amdgcn_sched_barrier(0);
       f = mfma_16b<T>(corr_k, corr_q, f);
       __builtin_amdgcn_sched_barrier(0);
