@@ -101,6 +101,20 @@ def test_cpu_tensors_are_refused_not_emulated(qfa):
         qfa.quant_flash_attn_qkv(x, x, x, False, 0.125)
     with pytest.raises(ValueError):
         qfa.asymmetric_quant_per_token(torch.randn(16, 64))
+    codes = torch.zeros(1, 2, 16, 64, dtype=torch.int8)
+    quant = (codes, torch.ones(1, 2, 16, 1, dtype=torch.float16), torch.zeros(1, 2, 16, 1, dtype=torch.int8))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        qfa.quant_flash_attn(x, x, quant, 0.125)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        qfa.quant_flash_attn_quantized_kv(x, x, x, quant, quant, True, 0.125)
+
+
+def test_routing_of_the_reference_entry_point():
+    """quant_flash_attn gives query blocks up to the measured crossover to the shared-KV kernels: 512 tokens,
+    1024 at head_dim 256 (where the INT8-score kernels run one wave per SIMD)."""
+    from quant_flash_attn_amd.quant_flash_attn import SHARED_KV_MAX_Q, shared_kv_max_q
+    assert SHARED_KV_MAX_Q == 512
+    assert shared_kv_max_q(64) == 512 and shared_kv_max_q(128) == 512 and shared_kv_max_q(256) == 1024
 
 
 def test_missing_library_fails_loudly(monkeypatch):
