@@ -188,7 +188,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   const int v_off = v_row * SM::VSTR + ((VSW::swz(v_row) + 2 * ((lane / 16) % 2) + (lane % 4) / 2) << 4) +
                     8 * (lane % 2);                                      // XOR with 64*db selects the d block
   // S^T block nb (32 keys) of the tile held in K buffer `buf`, for this wave's 32 queries
-  auto qk_block = [&](int buf, int nb, i32x16 &s) {
+  auto qk_block = [&](int buf, int nb, i32x16 &s) __attribute__((always_inline)) {
     const unsigned char *ks_ = smem + SM::OFF_K + buf * SM::K_BYTES;
 #pragma unroll
     for (int v = 0; v < 16; ++v) s[v] = 0;
@@ -212,7 +212,8 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   float l_run = 0.f;         // this lane's share of the row sum
 
   // raw int32 block -> u = sk * (S + zero-point correction); returns the block maximum of the row
-  auto prep = [&](int cbuf, int nb, const i32x16 &s, float (&u)[16], int j0, auto masked_tag) -> float {
+  auto prep = [&](int cbuf, int nb, const i32x16 &s, float (&u)[16], int j0, auto masked_tag)
+                  __attribute__((always_inline)) -> float {
     constexpr bool MASKED = decltype(masked_tag)::value;
     const unsigned char *cb = smem + SM::OFF_C + cbuf * SM::C_BYTES;
     const float *skp = reinterpret_cast<const float *>(cb);
@@ -243,7 +244,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   // move the reference maximum only when some row of the wave outgrew it by > 2^threshold
   // (the test is one compare against m_ref + threshold / a_i, kept in m_bound: it sits at the end
   // of a dependent chain that nothing else in the wave can overlap)
-  auto move_ref = [&](float mt) {
+  auto move_ref = [&](float mt) __attribute__((always_inline)) {
     {
       const float m_new = fmaxf(m_ref, mt);
       const float alpha = __builtin_amdgcn_exp2f(a_i * (m_ref - m_new));
@@ -257,11 +258,11 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
         for (int v = 0; v < 16; ++v) oacc[db][v] *= alpha;
     }
   };
-  auto rescale_if_needed = [&](float mt) {
+  auto rescale_if_needed = [&](float mt) __attribute__((always_inline)) {
     if (__builtin_amdgcn_ballot_w64(mt > m_bound) != 0) move_ref(mt);
   };
   // p = exp2(a_i*u - a_i*m_ref), packed; row sum; O^T += V^T . P^T for the 32 keys of block nb
-  auto exp_pv = [&](int vbuf, int nb, const float (&u)[16]) {
+  auto exp_pv = [&](int vbuf, int nb, const float (&u)[16]) __attribute__((always_inline)) {
     if (QK_ONLY) {   // keep the scores alive without exponentials or MFMAs
       float s = 0.f;
 #pragma unroll
@@ -375,7 +376,8 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
     // then kf is refilled from K block (kbuf, knb).
     // `copy(i)`, i = 0..2, is called between phases: the steady loop issues chunks of the next
     // tiles' copies there, so that the memory pipe sees a few requests at a time instead of a burst per tile
-    auto body = [&](int vbuf, auto nb_tag, int cbuf, int cnb, int kbuf, int knb, auto &&copy) {
+    auto body = [&](int vbuf, auto nb_tag, int cbuf, int cnb, int kbuf, int knb, auto &&copy)
+                    __attribute__((always_inline)) {
       static_assert(DB == 8 || DB == 4 || DB == 2, "fragment arrays are sized for head_dim 256, 128 or 64");
       u32x2 vr0[2 * DB], vr1[2 * DB];
       u32x4 pf0, pf1;
@@ -504,6 +506,36 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
       const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
       dma_wait();
       __syncthreads();
+    }
+    // ---- the wave's diagonal tile, as far as the pipeline has it already.  When the mask sits on a 32-key boundary
+    // (always with Nq == Nk) the tile holds one block cut by the diagonal, before it at most one block that is fully
+    // visible, behind it only invisible ones.  The scores of the tile's first block are in u, prepared by the last
+    // body; a visible first block goes through one more body, which also prepares the diagonal block.  The diagonal
+    // block then only needs the mask, the maximum and the P.V step: no score product is formed twice and the visible
+    // block keeps the pipelined pace (the generic loop below took 2 900 cycles per block where this takes 1 600).
+    if (!QK_ONLY && CAUSAL && D <= 128 && t < ntiles && coff % 32 == 0 && t == (q_first + coff + 1) / FWD_BN &&
+        (t + 1) * FWD_BN <= a.Nk) {
+      if (t + 2 < ntiles) load_k(t + 2, kb_free);
+      if (t + 1 < ntiles) load_v(t + 1);
+      const int j0 = t * FWD_BN;
+      const int nb_d = (q_first + coff - j0) / 32;   // 0 or 1, wave-uniform: the block that holds the diagonal
+      if (nb_d == 1) body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, no_copy);
+      float mt = -INFINITY;
+#pragma unroll
+      for (int aa = 0; aa < 4; ++aa)
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb) {
+          const int j = j0 + 32 * nb_d + 8 * aa + 4 * g + bb;
+          if (j > qi + coff) u[4 * aa + bb] = -INFINITY;
+          mt = fmaxf(mt, u[4 * aa + bb]);
+        }
+      rescale_if_needed(max_across_halves(mt));
+      exp_pv(t & 1, nb_d, u);
+      if (t + 2 < ntiles) store_k(kb_free);
+      const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
+      dma_wait();
+      __syncthreads();
+      ++t;
     }
   }
   // ---- masked tiles (diagonal, ragged end): one block at a time, nothing carried between blocks
