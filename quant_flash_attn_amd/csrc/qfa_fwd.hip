@@ -34,7 +34,11 @@
 //  * tiles without any masked score run a software-pipelined loop whose body is one straight
 //    basic block per 32-key block: exp2/pack of block b, the P.V MFMAs of block b, the INT8 MFMAs
 //    of block b+2 and the convert/correct/scale of block b+1 are independent of each other,
-//    so MFMA and VALU instructions interleave; diagonal and ragged tiles run a simple masked loop.
+//    so MFMA and VALU instructions interleave; ragged tiles run a simple masked loop, and so does the
+//    causal diagonal except where the pipeline already holds its scores (see the end of the pipelined part).
+//
+// Head dimensions 64, 128 and 256 are instances of the same code: three, two and one workgroup per CU (31, 58 and
+// 114 KB of LDS; 168, 250 and 256 + 256 registers per wave).
 //
 // V lies in LDS as it does in memory ([key][d] rows, 64-byte quarters XOR-swizzled against bank
 // conflicts) and is transposed on the way out: ds_read_b64_tr_b16 hands lane (d, k-group) four
