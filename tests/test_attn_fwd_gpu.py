@@ -196,8 +196,9 @@ def test_key_permutation_invariance(qfa):
     assert max_abs(o, o_p) <= 2e-2 and max_abs(lse, lse_p) < 2 * LSE_TOL   # O within two bf16 ulps of |O| <= 4
 
 
-def test_output_fully_written_and_deterministic(qfa):
-    q, k, v, _ = make_inputs("normal", 2, 2, 300, 128, seed=8)
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_output_fully_written_and_deterministic(qfa, D):
+    q, k, v, _ = make_inputs("normal", 2, 2, 300, D, seed=8)
     sm = 0.1
     qq = qfa.quantize_for_attention(q.to(DEV))
     kq = qfa.quantize_for_attention(k.to(DEV))
@@ -207,11 +208,19 @@ def test_output_fully_written_and_deterministic(qfa):
     assert not torch.isnan(o1.float()).any()
 
 
-def test_strided_qkv_layout(qfa):
-    """q, k, v stored [B,N,H,D] and passed as permuted views."""
-    B, H, N, D = 2, 3, 256, 64
+@pytest.mark.parametrize("D", [64, 256])
+def test_strided_qkv_layout(qfa, D):
+    """q, k, v stored [B,N,H,D] and passed as permuted views; forward and backward equal the contiguous run."""
+    B, H, N = 2, 3, 256
     q, k, v, _ = make_inputs("offset", B, H, N, D, seed=12)
     mk = lambda t: t.permute(0, 2, 1, 3).contiguous().to(DEV).permute(0, 2, 1, 3)
     o = qfa.quant_flash_attn_qkv(mk(q), mk(k), mk(v), True, 0.125)
     o_c = qfa.quant_flash_attn_qkv(q.to(DEV), k.to(DEV), v.to(DEV), True, 0.125)
     assert torch.equal(o, o_c)
+    ins = [mk(t).requires_grad_(True) for t in (q, k, v)]
+    ins_c = [t.to(DEV).requires_grad_(True) for t in (q, k, v)]
+    g = torch.randn(B, H, N, D, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).to(DEV)
+    qfa.quant_flash_attn_qkv(*ins, True, 0.125).backward(g)
+    qfa.quant_flash_attn_qkv(*ins_c, True, 0.125).backward(g)
+    for a, b in zip(ins, ins_c):
+        assert torch.equal(a.grad, b.grad)
