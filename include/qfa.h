@@ -77,6 +77,15 @@ int qfa_dequant_per_token(const int8_t *codes, const void *scale, int scale_dtyp
                           int64_t scn, int64_t sob, int64_t soh, int64_t son, void *stream);
 
 /*
+ * rowsum[b,h,n] = sum_d codes[b,h,n,d] (int32, dense [B*H*N]): the side output of qfa_quant_per_token, for
+ * codes that arrive already quantized.  qfa_attn_fwd / qfa_attn_bwd need it for the exact zero-point term of the
+ * INT8 score product; the reference has no counterpart (its kernels dequantize K before the product,
+ * quant_flash_attn.py:65).  D any multiple of 8 up to 256; codes 8-byte aligned, strides multiples of 8 bytes.
+ */
+int qfa_code_rowsum(const int8_t *codes, int32_t *rowsum, int64_t B, int64_t H, int64_t N, int D, int64_t scb,
+                    int64_t sch, int64_t scn, void *stream);
+
+/*
  * Attention forward on quantized Q and K:
  *     S = sm_scale * Q^ K^T,  Q^ = sq*(qc - zq),  K^ = sk*(kc - zk)   [causal: keep col <= row]
  *     O = softmax(S) V,   LSE = logsumexp(S) (natural log)

@@ -103,3 +103,20 @@ def dequantize_per_token(codes: torch.Tensor, scale: torch.Tensor, zero_point: t
             _lib.stream_of(codes))
     _lib.check(code, "qfa_dequant_per_token")
     return out
+
+
+def code_rowsum(codes: torch.Tensor) -> torch.Tensor:
+    """int32 [B,H,N,1] sum of each token's codes (what quantize_for_attention emits beside the codes), as a HIP
+    kernel, for codes that arrive already quantized."""
+    _lib.require_gpu(codes)
+    if codes.dim() != 4 or codes.dtype != torch.int8:
+        raise ValueError("codes must be a 4-D int8 tensor")
+    B, H, N, D = codes.shape
+    if codes.stride(3) != 1 or any(codes.stride(i) % 8 for i in range(3)) or codes.data_ptr() % 8:
+        codes = codes.contiguous()
+    out = torch.empty((B, H, N, 1), dtype=torch.int32, device=codes.device)
+    with torch.cuda.device(codes.device):
+        code = _lib.lib().qfa_code_rowsum(codes.data_ptr(), out.data_ptr(), B, H, N, D, codes.stride(0),
+                                          codes.stride(1), codes.stride(2), _lib.stream_of(codes))
+    _lib.check(code, "qfa_code_rowsum")
+    return out

@@ -84,6 +84,18 @@ int qfa_dequant_per_token(const int8_t *codes, const void *scale, int scale_dtyp
                         (hipStream_t)stream);
 }
 
+int qfa_code_rowsum(const int8_t *codes, int32_t *rowsum, int64_t B, int64_t H, int64_t N, int D, int64_t scb,
+                    int64_t sch, int64_t scn, void *stream) {
+  if (!codes || !rowsum) return set_error(QFA_EINVAL, "code_rowsum: null pointer");
+  if (B <= 0 || H <= 0 || N <= 0) return set_error(QFA_EINVAL, "code_rowsum: B, H, N must be positive");
+  if (D < 8 || D > 256 || D % 8 != 0)
+    return set_error(QFA_EUNSUPPORTED, "code_rowsum: head_dim %d is not a multiple of 8 between 8 and 256", D);
+  if (!aligned8(codes)) return set_error(QFA_EINVAL, "code_rowsum: codes must be 8-byte aligned");
+  if (scb <= 0 || sch <= 0 || scn < D || scb % 8 != 0 || sch % 8 != 0 || scn % 8 != 0)
+    return set_error(QFA_EINVAL, "code_rowsum: strides must be positive multiples of 8 bytes, token stride >= D");
+  return launch_rowsum(codes, rowsum, B, H, N, D, scb, sch, scn, (hipStream_t)stream);
+}
+
 static int check_attn_common(const char *who, const AttnArgs &a) {
   if (!a.qc || !a.sq || !a.zq || !a.rq || !a.kc || !a.sk || !a.zk || !a.rk || !a.v || !a.o || !a.lse)
     return set_error(QFA_EINVAL, "%s: null pointer argument", who);

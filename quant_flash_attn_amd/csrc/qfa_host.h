@@ -16,6 +16,8 @@ int check_launch(const char *what);
 int launch_quant(const void *x, int x_dtype, int8_t *codes, float *scale, void *scale_lp, int scale_lp_dtype,
                  int8_t *zp, int32_t *rowsum, int64_t B, int64_t H, int64_t N, int D, int64_t sxb, int64_t sxh,
                  int64_t sxn, int64_t scb, int64_t sch, int64_t scn, hipStream_t st);
+int launch_rowsum(const int8_t *codes, int32_t *rowsum, int64_t B, int64_t H, int64_t N, int D, int64_t scb,
+                  int64_t sch, int64_t scn, hipStream_t st);
 int launch_dequant(const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp, void *out,
                    int out_dtype, int64_t B, int64_t H, int64_t N, int D, int64_t scb, int64_t sch, int64_t scn,
                    int64_t sob, int64_t soh, int64_t son, hipStream_t st);

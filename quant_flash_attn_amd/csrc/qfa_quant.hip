@@ -324,4 +324,58 @@ int launch_dequant(const int8_t *codes, const void *scale, int scale_dtype, cons
   return set_error(QFA_EINVAL, "dequant: bad out_dtype");
 }
 
+// ---------------------------------------------------------------------------------------------
+// Row sums of given codes: rowsum[t] = sum_d codes[t][d], the side output the quantizer emits, for codes that
+// arrive already quantized (the zero-point term of the INT8 score product needs them).
+struct RowsumArgs {
+  const int8_t *codes;
+  int32_t *rowsum;
+  int64_t N, H;
+  int64_t scb, sch, scn;
+  int chunks_per_bh;
+  int D;
+};
+
+template <int DP> __global__ __launch_bounds__(256) void rowsum_kernel(RowsumArgs a) {
+  constexpr int LPT = DP / 8;
+  constexpr int TPP = 256 / LPT;
+  const int tid = threadIdx.x;
+  const int sub = tid % LPT;
+  const int64_t bh = blockIdx.x / a.chunks_per_bh;
+  const int64_t chunk = blockIdx.x % a.chunks_per_bh;
+  const int64_t b = bh / a.H, h = bh % a.H;
+  const int64_t n = chunk * (int64_t)TPP + tid / LPT;
+  const int64_t nn = n < a.N ? n : a.N - 1;          // every lane takes part in the reduction
+  int sum = 0;
+  if (sub * 8 < a.D) {
+    u32x2 w = *reinterpret_cast<const u32x2 *>(a.codes + b * a.scb + h * a.sch + nn * a.scn + sub * 8);
+    w[0] ^= 0x80808080u;                               // biased bytes: code + 128
+    w[1] ^= 0x80808080u;
+    sum = (int)__builtin_amdgcn_sad_u8(w[0], 0u, 0u);
+    sum = (int)__builtin_amdgcn_sad_u8(w[1], 0u, (unsigned)sum) - 8 * 128;
+  }
+  sum = group_sum<LPT>(sum);
+  if (n < a.N && sub == 0) a.rowsum[bh * a.N + n] = sum;
+}
+
+int launch_rowsum(const int8_t *codes, int32_t *rowsum, int64_t B, int64_t H, int64_t N, int D, int64_t scb,
+                  int64_t sch, int64_t scn, hipStream_t st) {
+  if (D < 8 || D > 256 || D % 8 != 0) return set_error(QFA_EUNSUPPORTED, "code_rowsum: head_dim must be a multiple of 8, at most 256");
+  RowsumArgs a;
+  a.codes = codes; a.rowsum = rowsum; a.N = N; a.H = H; a.scb = scb; a.sch = sch; a.scn = scn; a.D = D;
+  const int DP = padded_head_dim(D);
+  const int tpp = 256 / (DP / 8);
+  const int64_t chunks = (N + tpp - 1) / tpp;
+  if (chunks * B * H > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "code_rowsum: too many tokens for one launch");
+  a.chunks_per_bh = (int)chunks;
+  const dim3 grid((unsigned)(chunks * B * H)), block(256);
+  switch (DP) {
+    case 32: rowsum_kernel<32><<<grid, block, 0, st>>>(a); break;
+    case 64: rowsum_kernel<64><<<grid, block, 0, st>>>(a); break;
+    case 128: rowsum_kernel<128><<<grid, block, 0, st>>>(a); break;
+    default: rowsum_kernel<256><<<grid, block, 0, st>>>(a); break;
+  }
+  return check_launch("qfa_code_rowsum");
+}
+
 }  // namespace qfa

@@ -23,7 +23,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from .asymmetric_quant import QuantizedTokens, dequantize_per_token, quantize_for_attention
+from .asymmetric_quant import QuantizedTokens, code_rowsum, dequantize_per_token, quantize_for_attention
 
 _IO_DTYPES = (torch.bfloat16, torch.float16)
 
@@ -278,7 +278,7 @@ class QuantFlashAttnQuantizedKV(torch.autograd.Function):
             raise ValueError(f"shape mismatch: q {tuple(q.shape)}, k codes {tuple(kc.shape)}, v codes {tuple(vc.shape)}")
         io = _io_dtype(q)
         qq = quantize_for_attention(q)
-        kq = QuantizedTokens(kc, ks.to(torch.float32), kz, kc.sum(dim=-1, keepdim=True, dtype=torch.int32))
+        kq = QuantizedTokens(kc, ks.to(torch.float32), kz, code_rowsum(kc))
         v16 = dequantize_per_token(vc, vs, vz, io)
         o, lse = attn_fwd_quantized(qq, kq, v16, causal, sm_scale)
         ctx.save_for_backward(*qq, *kq, v16, o, lse)
@@ -367,7 +367,7 @@ def _legacy_operands(q, codes, scale, zp, io):
     """Operands of the INT8-score kernels for the reference's entry point: Q quantized per token,
     K = the caller's codes with the scale exactly as stored, V = dequant(kv) (quant_flash_attn.py:65)."""
     qq = quantize_for_attention(q)
-    kq = QuantizedTokens(codes, scale.to(torch.float32), zp, codes.sum(dim=-1, keepdim=True, dtype=torch.int32))
+    kq = QuantizedTokens(codes, scale.to(torch.float32), zp, code_rowsum(codes))
     return qq, kq, dequantize_per_token(codes, scale, zp, io)
 
 

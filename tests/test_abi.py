@@ -67,6 +67,9 @@ def test_argument_errors_need_no_gpu(qfa):
     assert rc == -2 and b"2^28" in L.qfa_last_error()
     rc = L.qfa_bwd_delta(None, ok_ptr, ok_ptr, 2, 1, 1, 8, 64, 512, 512, 64, 512, 512, 64, None)
     assert rc == -1
+    assert L.qfa_code_rowsum(None, ok_ptr, 1, 1, 8, 64, 512, 512, 64, None) == -1
+    assert L.qfa_code_rowsum(ok_ptr, ok_ptr, 1, 1, 8, 44, 512, 512, 64, None) == -2 and b"head_dim" in L.qfa_last_error()
+    assert L.qfa_code_rowsum(ok_ptr, ok_ptr, 1, 1, 8, 64, 512, 512, 60, None) == -1 and b"strides" in L.qfa_last_error()
     # backward scratch: one blob per 64-row tile (32-row at head_dim 256) and side; nothing for other widths
     ws = L.qfa_attn_bwd_workspace_bytes
     assert ws(1, 1, 64, 64, 64) == 2 * 64 * 64 * 2 + (5 + 3) * 64 * 4

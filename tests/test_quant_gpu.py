@@ -113,6 +113,20 @@ def test_dequantize_kernel(qfa):
     assert torch.equal(out16.cpu(), ref16.to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("D", [8, 64, 96, 128, 200, 256])
+def test_code_rowsum_kernel(qfa, D):
+    """Row sums of given codes (qfa_code_rowsum): equal to the integer sum, on contiguous and on strided codes."""
+    g = torch.Generator().manual_seed(D)
+    codes = torch.randint(-128, 128, (2, 3, 133, D), generator=g, dtype=torch.int8)
+    codes[0, 0, 0] = 127
+    codes[0, 0, 1] = -128
+    got = qfa.code_rowsum(codes.to(DEV))
+    want = codes.to(torch.int32).sum(-1, keepdim=True)
+    assert got.dtype == torch.int32 and got.shape == (2, 3, 133, 1) and torch.equal(got.cpu(), want)
+    strided = codes.permute(0, 2, 1, 3).contiguous().to(DEV).permute(0, 2, 1, 3)      # [B,N,H,D] storage
+    assert torch.equal(qfa.code_rowsum(strided).cpu(), want)
+
+
 def test_outputs_fully_written_and_deterministic(qfa):
     q, _, _, _ = make_inputs("normal", 1, 3, 1000, 64, seed=6)
     xg = q.to(DEV)
