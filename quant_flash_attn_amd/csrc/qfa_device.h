@@ -63,6 +63,20 @@ template <> __device__ __forceinline__ float dot2_ones<_Float16>(unsigned w, flo
   return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), ones, c, false);
 }
 
+// The same sum written to a NEW register (the three-operand encoding; the compiler only forms the accumulate-in-place
+// one and would copy c first): for a chain that starts from a value which must survive
+template <typename T> __device__ __forceinline__ float dot2_ones_keep(unsigned w, float c);
+template <> __device__ __forceinline__ float dot2_ones_keep<__bf16>(unsigned w, float c) {
+  float r;
+  asm("v_dot2_f32_bf16 %0, %1, %2, %3" : "=v"(r) : "v"(w), "s"(0x3f803f80u), "v"(c));
+  return r;
+}
+template <> __device__ __forceinline__ float dot2_ones_keep<_Float16>(unsigned w, float c) {
+  float r;
+  asm("v_dot2_f32_f16 %0, %1, %2, %3" : "=v"(r) : "v"(w), "s"(0x3c003c00u), "v"(c));
+  return r;
+}
+
 // ---- MFMA wrappers (A and B: 16 bytes per lane; C/D: 16 dwords per lane) ------------------------
 // 32x32x32 int8:  A lane l = row l%32, 16 consecutive k at k-group l/32;  B lane l = column l%32,
 // same k slots;  D lane l = column l%32, register v = row 8*(v/4) + 4*(l/32) + v%4.
@@ -78,6 +92,17 @@ template <> __device__ __forceinline__ f32x16 mfma_16b<__bf16>(u32x4 a, u32x4 b,
 template <> __device__ __forceinline__ f32x16 mfma_16b<_Float16>(u32x4 a, u32x4 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
                                                 0);
+}
+
+// 32x32x8, the older 16-bit shape (A and B: 4 elements = 8 bytes per lane, k-group l/32 holds k = 4g..4g+3): the same
+// 32 cycles on the matrix pipe as the x16 shape, half the operand registers -- for products of rank <= 8
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+template <typename T> __device__ __forceinline__ f32x16 mfma_16b_k8(u32x2 a, u32x2 b, f32x16 c);
+template <> __device__ __forceinline__ f32x16 mfma_16b_k8<__bf16>(u32x2 a, u32x2 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ f32x16 mfma_16b_k8<_Float16>(u32x2 a, u32x2 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
 }
 
 // ---- lane exchanges ---------------------------------------------------------------------------

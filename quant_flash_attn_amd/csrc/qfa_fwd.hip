@@ -112,7 +112,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   const float a_i = a.sq[tq0 + qi_c] * a.sm_scale_log2;        // > 0
   // query side of the rank-4 correction: k-group 0 multiplies the two digits of rk by -zq,
   // k-group 1 multiplies zk (stored twice) by minus the two digits of c = rq - D*zq
-  u32x4 corr_q = {0u, 0u, 0u, 0u};
+  u32x2 corr_q = {0u, 0u};
   {
     // two digits of 7 bits each (|c| <= 32640) up to head_dim 128, of 8 bits at head_dim 256 (|c| <= 65280): either
     // way each digit, shifted into place, has at most 8 significant bits and is exact in the 16-bit type
@@ -171,10 +171,11 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
     if (tid < FWD_BN) {
       unsigned char *cb = smem + SM::OFF_C + buf * SM::C_BYTES;
       reinterpret_cast<float *>(cb)[tid] = c_sk;
-      u32x2 dg;
+      // the A operand of the correction product as it is read: per k-group a pair of 16-bit values and a zero dword
+      u32x4 dg = {0u, 0u, 0u, 0u};
       dg[0] = base128_pair<T>(c_rk);                      // k-group 0: digits of rk
-      dg[1] = pack2<T>((float)c_zk, (float)c_zk);         // k-group 1: zk, zk
-      reinterpret_cast<u32x2 *>(cb + FWD_BN * 4)[tid] = dg;
+      dg[2] = pack2<T>((float)c_zk, (float)c_zk);         // k-group 1: zk, zk
+      reinterpret_cast<u32x4 *>(cb + FWD_BN * 4)[tid] = dg;
     }
   };
   auto load_v = [&](int t) {
@@ -221,12 +222,12 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
     constexpr bool MASKED = decltype(masked_tag)::value;
     const unsigned char *cb = smem + SM::OFF_C + cbuf * SM::C_BYTES;
     const float *skp = reinterpret_cast<const float *>(cb);
-    const unsigned *dgp = reinterpret_cast<const unsigned *>(cb + FWD_BN * 4);
+    const u32x2 *dgp = reinterpret_cast<const u32x2 *>(cb + FWD_BN * 4);
     f32x16 f;
 #pragma unroll
     for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
-    u32x4 corr_k = {dgp[2 * (32 * nb + lr) + g], 0u, 0u, 0u};
-    f = mfma_16b<T>(corr_k, corr_q, f);
+    const u32x2 corr_k = dgp[2 * (32 * nb + lr) + g];
+    f = mfma_16b_k8<T>(corr_k, corr_q, f);
     float mt = -INFINITY;
 #pragma unroll
     for (int aa = 0; aa < 4; ++aa) {
@@ -350,31 +351,36 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
         vr[2 * db + 1] = lds_read_tr16_async<ROW0 + 8 * SM::VSTR>(ad);
       }
     };
-    auto exp_half = [&](int hh, u32x4 &pf, float &lsum) {
-      lsum = 0.f;
+    // lnew = l_run + the 8 probabilities (the running sum continues in a second register, so that l_run is still
+    // there if the probabilities have to be formed again)
+    auto exp_half = [&](int hh, u32x4 &pf, float &lnew) {
+      float l = l_run;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, u[8 * hh + 2 * e], nm));
         const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(a_i, u[8 * hh + 2 * e + 1], nm));
         pf[e] = pack2<T>(p0, p1);
-        lsum = dot2_ones<T>(pf[e], lsum);   // sum of the rounded pair, fp32 accumulate
+        l = e == 0 ? dot2_ones_keep<T>(pf[e], l) : dot2_ones<T>(pf[e], l);   // sum of the rounded pair, fp32 accumulate
       }
+      lnew = l;
     };
     // The pipelined loop takes no running maximum.  The probabilities of 16 keys are formed against the
-    // current reference and their sum is looked at before they reach the P.V MFMAs: only if some lane's
-    // sum left the range below (a score outgrew the reference by more than 2^60, or overflowed) is the
+    // current reference and the running sum is looked at before they reach the P.V MFMAs: only if some lane's
+    // sum left the range below (scores outgrew the reference by about 2^60, or overflowed) is the
     // maximum of the block taken, the reference moved (O and the row sum rescaled) and the 16
-    // probabilities formed again.  Any reference gives the same O after the final division.
+    // probabilities formed again.  Any reference gives the same O after the final division.  The reference
+    // moves at least far enough to bring the sum so far back to order one (a sum that crept up to the limit
+    // through many terms is not brought down by the maximum of the current block alone).
     constexpr float SUM_LIMIT = 0x1p60f;
-    auto check_half = [&](int hh, u32x4 &pf, float &lsum) {
-      if (__builtin_amdgcn_ballot_w64(!(lsum <= SUM_LIMIT)) != 0) {
-        float mt = -INFINITY;
+    auto check_half = [&](int hh, u32x4 &pf, float &lnew) {
+      if (__builtin_amdgcn_ballot_w64(!(lnew <= SUM_LIMIT)) != 0) {
+        float mt = m_ref + __log2f(fmaxf(l_run, 1.0f)) / a_i;
 #pragma unroll
         for (int v = 8 * hh; v < 16; ++v) mt = fmaxf(mt, u[v]);   // first half: the whole block
         move_ref(max_across_halves(mt));
-        exp_half(hh, pf, lsum);
+        exp_half(hh, pf, lnew);
       }
-      l_run += lsum;
+      l_run = lnew;
     };
     // one body: V block (vbuf, nb); scores of the next block from kf; its constants in (cbuf, cnb);
     // then kf is refilled from K block (kbuf, knb).
@@ -415,7 +421,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa)
         sk4[aa] = *reinterpret_cast<const f32x4 *>(cb + (32 * cnb + 8 * aa + 4 * g) * 4);
-      const u32x4 corr_k = {reinterpret_cast<const unsigned *>(cb + FWD_BN * 4)[2 * (32 * cnb + lr) + g], 0u, 0u, 0u};
+      const u32x2 corr_k = reinterpret_cast<const u32x2 *>(cb + FWD_BN * 4)[2 * (32 * cnb + lr) + g];
       __builtin_amdgcn_sched_barrier(0);
       // P.V of the first 16 keys under the exponentials of the second 16 and the conversion of the next
       // block's raw scores; their zero-point correction (one MFMA) goes last, so that its result has the
@@ -437,7 +443,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
 #pragma unroll
       for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
       __builtin_amdgcn_sched_barrier(0);
-      f = mfma_16b<T>(corr_k, corr_q, f);
+      f = mfma_16b_k8<T>(corr_k, corr_q, f);
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(0);
       if (!QK_ONLY) {

@@ -31,7 +31,7 @@ template <int D> struct FwdSmem {
   static constexpr int VSTR = 2 * D;             // bytes per V row (dense, quarters swizzled: SwzQuad<2D>)
   static constexpr int K_BYTES = FWD_BN * KSTR;
   static constexpr int V_BYTES = FWD_BN * VSTR;
-  static constexpr int C_BYTES = FWD_BN * 4 + FWD_BN * 8;  // key scale; correction digits (2 dwords/key)
+  static constexpr int C_BYTES = FWD_BN * 4 + FWD_BN * 16;  // key scale; correction operands (per key and k-group a pair and a zero dword)
   static constexpr int OFF_K = 0;                     // 3 buffers
   static constexpr int OFF_V = 3 * K_BYTES;           // 2 buffers
   static constexpr int OFF_C = OFF_V + 2 * V_BYTES;   // 3 buffers
