@@ -137,6 +137,7 @@ template <int ROW_BYTES> struct Swz {
   static constexpr int CPR = ROW_BYTES / 16;                 // chunks per row (4, 8, 16 or 32)
   static constexpr int RP = CPR >= 16 ? 1 : 16 / CPR;        // rows per 256 bytes (1 for rows of one or more lines)
   static constexpr int MOD = CPR >= 16 ? 16 : CPR;           // only the slot inside the 256-byte line matters
+  static constexpr int PERIOD = RP * MOD;                    // swz(row + PERIOD) == swz(row)
   static __device__ __forceinline__ int swz(int row) { return (row / RP) % MOD; }
   // byte offset of logical chunk c of row r inside the tile
   static __device__ __forceinline__ int off(int r, int c) { return r * ROW_BYTES + ((c ^ swz(r)) << 4); }
@@ -159,6 +160,7 @@ template <int ROW_BYTES> struct SwzQuad {
   static constexpr int CPR = ROW_BYTES / 16;
   static constexpr int RPL = ROW_BYTES >= 256 ? 1 : 256 / ROW_BYTES;   // rows per 256-byte line
   static constexpr int QPR = ROW_BYTES >= 256 ? 4 : ROW_BYTES / 64;      // quarters the XOR moves over (one line at most)
+  static constexpr int PERIOD = RPL * QPR;                               // swz(row + PERIOD) == swz(row)
   static __device__ __forceinline__ int swz(int row) { return 4 * ((row / RPL) % QPR); }
 };
 
@@ -218,6 +220,32 @@ template <int ROW_BYTES, int ROWS, int NT, typename S = Swz<ROW_BYTES>> struct T
     for (int i = 0; i < N; ++i)
       if (TOTAL % NT == 0 || tid + NT * i < TOTAL)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lptr_t)(lds + (wave_u * 64 + NT * i) * 16), 16, (int)off[i], 0, 0, 0);
+  }
+};
+// TileCopy for tiles whose chunks all look alike from a thread's point of view: chunk i of a thread lies
+// i * (NT / CPR) rows below its chunk 0 at the same swizzled position (the rows per chunk are a multiple of the
+// swizzle's period), so ONE per-thread offset serves every chunk and the step goes into the scalar offset of the load.
+template <int ROW_BYTES, int ROWS, int NT, typename S = Swz<ROW_BYTES>> struct TileCopyU {
+  static constexpr int TOTAL = ROWS * S::CPR;
+  static constexpr int N = TOTAL / NT;
+  static constexpr int RPC = NT / S::CPR;   // rows per chunk
+  static_assert(TOTAL % NT == 0 && NT % S::CPR == 0 && RPC % S::PERIOD == 0, "chunks must repeat the swizzle");
+  unsigned off0;    // per thread
+  unsigned step;    // uniform: bytes between a thread's consecutive chunks
+  __device__ __forceinline__ void init(unsigned gstride, int tid) {
+    const int row = tid / S::CPR, pos = tid % S::CPR;
+    off0 = (unsigned)row * gstride + (unsigned)((pos ^ S::swz(row)) << 4);
+    step = (unsigned)RPC * gstride;
+  }
+  // chunk i (a compile-time constant at the call site) of a copy through the descriptor of the tile's first row
+  __device__ __forceinline__ void issue_one(rsrc_t rs, unsigned char *lds, int wave_u, int i) const {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lptr_t)(lds + (wave_u * 64 + NT * i) * 16), 16, (int)off0,
+                                             (int)(step * (unsigned)i), 0, 0);
+  }
+  __device__ __forceinline__ void issue(const void *tile_base, unsigned char *lds, int wave_u) const {
+    const rsrc_t rs = make_rsrc(tile_base, 0x7fffffffu);
+#pragma unroll
+    for (int i = 0; i < N; ++i) issue_one(rs, lds, wave_u, i);
   }
 };
 // dense swizzle-free layout for TileCopy (contiguous bytes)

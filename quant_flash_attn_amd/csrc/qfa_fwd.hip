@@ -4,7 +4,8 @@
 // Work split.  One workgroup = 4 waves = 128 query rows of one (batch, head) (8 waves per workgroup
 // halve the tile copies per query but measured 9 % slower: the barrier then waits for the slowest of
 // 8 waves); each wave owns
-// 32 queries.  K (3 buffers) and V (2 buffers) stream through LDS in tiles of 64 keys, copied by
+// 32 queries.  K, V and the per-key constants stream through LDS in tiles of 64 keys, three buffers each
+// (tile t in buffer t % 3), copied by
 // direct global->LDS loads (no staging registers, no address or repacking work on the vector
 // pipe); K and the per-key constants are resident one tile ahead of V because the score product
 // runs ahead.
@@ -19,26 +20,40 @@
 // Zero points.  With integer codes,  sum_d (qc-zq)(kc-zk) = A - zq*rk - zk*(rq - D*zq), A the int32
 // MFMA result and rq, rk the code row sums.  The correction is a rank-4 update with integer
 // entries of at most 8 significant bits (rk and rq - D*zq split into two digits), so it runs as ONE extra 16-bit
-// MFMA on the converted accumulator instead of per-score VALU work; every product and partial sum
+// MFMA instead of per-score VALU work; every product and partial sum
 // is an integer below 2^24, hence exact in fp32.  Then one multiply by the key scale; the query
 // scale, sm_scale and log2(e) are folded into the exp2 argument.
 //
-// The kernel is bound by softmax VALU work, not by MFMA, so the design goal is to keep the vector
-// pipe busy and hide the matrix pipe under it:
+// What bounds the kernel is the issue rate of the vector pipe (every vector instruction takes about 4.5
+// cycles of it with two waves per SIMD and an MFMA about twice that, whatever else overlaps), so the design goal is
+// the smallest number of vector instructions per score:
 //  * the reference maximum is only moved (and O rescaled) when it has to be (any reference gives the
 //    same O after the final division): the masked loop moves it when a row exceeds it by more than
-//    2^8, the pipelined loop takes no maximum at all and watches the sum of each 16 probabilities
-//    instead (one compare; see check_half), so the rescale is a rare branch instead of 64 multiplies
+//    2^8, the pipelined loop takes no maximum at all and watches the running sum of the probabilities
+//    instead (one compare per 16 keys; see check_half), so the rescale is a rare branch instead of 64 multiplies
 //    and 8 maxima per block;
 //  * row sums are taken over packed pairs with v_dot2;
+//  * the int32 -> fp32 conversion of the scores is done by the matrix pipe (see "biased accumulators" below);
+//  * the hot loop is unrolled over three tiles, so that every LDS address in it is a loop-invariant register plus
+//    an immediate offset;
 //  * tiles without any masked score run a software-pipelined loop whose body is one straight
 //    basic block per 32-key block: exp2/pack of block b, the P.V MFMAs of block b, the INT8 MFMAs
-//    of block b+2 and the convert/correct/scale of block b+1 are independent of each other,
+//    of block b+2 and the correct/scale of block b+1 are independent of each other,
 //    so MFMA and VALU instructions interleave; ragged tiles run a simple masked loop, and so does the
 //    causal diagonal except where the pipeline already holds its scores (see the end of the pipelined part).
 //
-// Head dimensions 64, 128 and 256 are instances of the same code: three, two and one workgroup per CU (31, 58 and
-// 114 KB of LDS; 168, 250 and 256 + 256 registers per wave).
+// Biased accumulators.  The correction MFMA runs FIRST, from a zero accumulator, with one more product term that
+// adds c0 = 1.5 * 2^23: its fp32 result c0 + corr lies in [2^23, 2^24), where consecutive floats are consecutive
+// integers and the bit pattern is 0x4B000000 + (value - 2^23).  The INT8 MFMAs then accumulate A onto that BIT
+// PATTERN (integer adds), which read as a float is c0 + corr + A = c0 + S exactly, as long as it stays inside the
+// binade; a third small MFMA adds -c0 and leaves the integer score S as an fp32 number.  Sixteen v_cvt_f32_i32 per
+// block become one MFMA.  The two range conditions (|corr| and |S| below 2^22, intermediate sums of the first
+// MFMA below 2^24 in any order) are checked per query in the prologue from quantities the wave has anyway
+// (|zq|, |rq - D zq| and sum_d |qc_d - zq|, bounded against the worst key); a wave with a query that could leave
+// the window -- rows pinned at one end of the code range -- takes the masked loop, which converts explicitly, for
+// all its tiles.
+//
+// Head dimensions 64, 128 and 256 are instances of the same code: three, two and one workgroup per CU.
 //
 // V lies in LDS as it does in memory ([key][d] rows, 64-byte quarters XOR-swizzled against bank
 // conflicts) and is transposed on the way out: ds_read_b64_tr_b16 hands lane (d, k-group) four
@@ -51,6 +66,10 @@
 
 namespace qfa {
 
+template <typename X> struct is_static_int : std::false_type {};
+template <int V> struct is_static_int<std::integral_constant<int, V>> : std::true_type {};
+template <int V> using ic = std::integral_constant<int, V>;
+
 // QK_ONLY is the measurement variant of the same kernel: identical loads, INT8 product, zero-point
 // correction, scaling and running maximum, with the exponentials and the P.V product compiled out
 // (it writes the scaled row maximum where the LSE would go and leaves O untouched).  It exists to
@@ -62,7 +81,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   typedef FwdSmem<D> SM;
   constexpr int KS = D / 32;   // int8 k-steps of 32
   constexpr int DB = D / 32;   // 32-row blocks of O^T
-  __shared__ __attribute__((aligned(16))) unsigned char smem[SM::TOTAL];
+  __shared__ __attribute__((aligned(256))) unsigned char smem[SM::TOTAL];
 
   // ---- block -> (batch*head, query block); consecutive ids of one XCD share a head's K/V in its L2
   const int L = blockIdx.x;
@@ -110,18 +129,40 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
     qf[ks] = *reinterpret_cast<const i32x4 *>(qc_bh + (int64_t)qi_c * a.sqn + ks * 32 + g * 16);
   const int zq_i = (int)a.zq[tq0 + qi_c];
   const float a_i = a.sq[tq0 + qi_c] * a.sm_scale_log2;        // > 0
-  // query side of the rank-4 correction: k-group 0 multiplies the two digits of rk by -zq,
-  // k-group 1 multiplies zk (stored twice) by minus the two digits of c = rq - D*zq
-  u32x2 corr_q = {0u, 0u};
+  // Query side (B operand) of the correction product, 4 k-slots per k-group: k-group 0 multiplies the two digits of
+  // rk by -zq and the constant 2^11 by 3*2^11 (= c0, the bias of the pipelined loop); k-group 1 multiplies zk
+  // (stored twice) by minus the two digits of c = rq - D*zq.
+  // Two digits of 7 bits each (|c| <= 32640) up to head_dim 128, of 8 bits at head_dim 256 (|c| <= 65280): either
+  // way each digit, shifted into place, has at most 8 significant bits and is exact in the 16-bit type.
+  constexpr int SH = D > 128 ? 8 : 7;
+  const int c_i = a.rq[tq0 + qi_c] - D * zq_i;
+  u32x2 corr_q;
   {
-    // two digits of 7 bits each (|c| <= 32640) up to head_dim 128, of 8 bits at head_dim 256 (|c| <= 65280): either
-    // way each digit, shifted into place, has at most 8 significant bits and is exact in the 16-bit type
-    constexpr int SH = D > 128 ? 8 : 7;
-    const int c = a.rq[tq0 + qi_c] - D * zq_i;
-    const int hi = c >> SH, lo = c & ((1 << SH) - 1);
+    const int hi = c_i >> SH, lo = c_i & ((1 << SH) - 1);
     corr_q[0] = g == 0 ? pack2<T>((float)(-zq_i), (float)(-zq_i)) : pack2<T>((float)(-(hi * (1 << SH))), (float)(-lo));
+    corr_q[1] = g == 0 ? pack2<T>(6144.0f, 0.0f) : 0u;
   }
+  // A operand that takes the bias out again: -2^11 in the slot that meets 3*2^11
+  const u32x2 unbias_a = {0u, g == 0 ? pack2<T>(-2048.0f, 0.0f) : 0u};
   const int q_first = m0 + wave * 32, q_last = q_first + 31;
+
+  // ---- may this wave's queries use biased accumulators (see the head of the file)?  For every key:
+  //   |terms of the first MFMA| <= |zq| (128 D + 127) + 128 (|c| + 2 * 2^SH) =: tq   (|rk digit sum| <= 128 D + 127, |zk| <= 128)
+  //   |S| <= 255 * sum_d |qc_d - zq| =: 255 mq
+  // and both must stay below 2^22.
+  bool bias_ok;
+  {
+    const unsigned zb = ((unsigned)(zq_i + 128) & 0xffu) * 0x01010101u;
+    unsigned mq = 0;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) mq = __builtin_amdgcn_sad_u8((unsigned)qf[ks][j] ^ 0x80808080u, zb, mq);
+    mq += (unsigned)__shfl_xor((int)mq, 32, 64);
+    const unsigned tq = (unsigned)abs(zq_i) * (128u * D + 127u) + 128u * ((unsigned)abs(c_i) + (2u << SH));
+    const bool ok = 255u * mq < (1u << 22) && tq < (1u << 22);
+    bias_ok = __builtin_amdgcn_ballot_w64(!ok) == 0;
+  }
 
   // ---- tile range
   int kv_end = a.Nk;
@@ -137,10 +178,10 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   float c_sk;
   int c_rk, c_zk;
 
-  // Full tiles: per-thread chunk offsets computed once (TileCopy); ragged tiles (rows clamped to the
+  // Full tiles: one per-thread offset for all chunks (TileCopyU); ragged tiles (rows clamped to the
   // last key) take the generic path.
-  TileCopy<D, FWD_BN, NT, KSW> cp_k;
-  TileCopy<2 * D, FWD_BN, NT, VSW> cp_v;
+  TileCopyU<D, FWD_BN, NT, KSW> cp_k;
+  TileCopyU<2 * D, FWD_BN, NT, VSW> cp_v;
   cp_k.init((unsigned)a.skn, tid);
   cp_v.init((unsigned)(a.svn * sizeof(T)), tid);
 
@@ -162,7 +203,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
     const int j0 = t * FWD_BN;
     unsigned char *dst = smem + SM::OFF_K + buf * SM::K_BYTES;
     if (j0 + FWD_BN <= a.Nk)
-      cp_k.issue(reinterpret_cast<const unsigned char *>(kc_bh) + (int64_t)j0 * a.skn, dst, wave_u, tid);
+      cp_k.issue(reinterpret_cast<const unsigned char *>(kc_bh) + (int64_t)j0 * a.skn, dst, wave_u);
     else
       dma_rows<D, FWD_BN, NT, KSW>(reinterpret_cast<const unsigned char *>(kc_bh), a.skn, j0, a.Nk - 1, dst, tid);
     load_kc(t);
@@ -171,38 +212,52 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
     if (tid < FWD_BN) {
       unsigned char *cb = smem + SM::OFF_C + buf * SM::C_BYTES;
       reinterpret_cast<float *>(cb)[tid] = c_sk;
-      // the A operand of the correction product as it is read: per k-group a pair of 16-bit values and a zero dword
+      // the A operand of the correction product as it is read: per k-group two dwords
       u32x4 dg = {0u, 0u, 0u, 0u};
-      dg[0] = base128_pair<T>(c_rk);                      // k-group 0: digits of rk
+      dg[0] = base128_pair<T>(c_rk);                      // k-group 0: digits of rk,
+      dg[1] = pack2<T>(2048.0f, 0.0f);                    //            and the constant that meets 3*2^11 (the bias c0)
       dg[2] = pack2<T>((float)c_zk, (float)c_zk);         // k-group 1: zk, zk
       reinterpret_cast<u32x4 *>(cb + FWD_BN * 4)[tid] = dg;
     }
   };
-  auto load_v = [&](int t) {
+  auto load_v = [&](int t, int buf) {
     const int j0 = t * FWD_BN;
-    unsigned char *dst = smem + SM::OFF_V + (t & 1) * SM::V_BYTES;
+    unsigned char *dst = smem + SM::OFF_V + buf * SM::V_BYTES;
     const int64_t vstride = a.svn * (int64_t)sizeof(T);
     if (j0 + FWD_BN <= a.Nk)
-      cp_v.issue(reinterpret_cast<const unsigned char *>(v_bh) + (int64_t)j0 * vstride, dst, wave_u, tid);
+      cp_v.issue(reinterpret_cast<const unsigned char *>(v_bh) + (int64_t)j0 * vstride, dst, wave_u);
     else
       dma_rows<2 * D, FWD_BN, NT, VSW>(reinterpret_cast<const unsigned char *>(v_bh), vstride, j0, a.Nk - 1, dst, tid);
   };
   // this lane's read offsets inside a tile (the swizzle terms only depend on the lane)
   const int k_swz = KSW::swz(lr);                                        // rows 32*nb + lr
+  int kq[KS];                                                            // K fragment ks of the lane's row
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) kq[ks] = lr * SM::KSTR + (((2 * ks + g) ^ k_swz) << 4);
   const int v_row = (lane % 16) / 4;                                     // source row of the transposing read
   const int v_off = v_row * SM::VSTR + ((VSW::swz(v_row) + 2 * ((lane / 16) % 2) + (lane % 4) / 2) << 4) +
                     8 * (lane % 2);                                      // XOR with 64*db selects the d block
+  unsigned vq[DB];                                                       // LDS address of the lane's V fragment of d block db
+#pragma unroll
+  for (int db = 0; db < DB; ++db) vq[db] = lds_addr(smem + SM::OFF_V) + 4 * g * SM::VSTR + (v_off ^ (64 * db));
+  const int c_skq = 16 * g;             // key scales of the lane's k-group inside a group of 8 keys
+  const int c_crq = (2 * lr + g) * 8;   // correction operand of (key lr, k-group g)
+  // the constants of block (buf, nb): key scales of keys 8aa + 4g + {0..3}, correction operand of key lr
+  auto sk_of = [&](auto buf, int nb, int aa) -> f32x4 {
+    return *reinterpret_cast<const f32x4 *>(smem + SM::OFF_C + (int)buf * SM::C_BYTES + (32 * nb + 8 * aa) * 4 + c_skq);
+  };
+  auto corr_of = [&](auto buf, int nb) -> u32x2 {
+    return *reinterpret_cast<const u32x2 *>(smem + SM::OFF_C + (int)buf * SM::C_BYTES + FWD_BN * 4 + 32 * nb * 16 + c_crq);
+  };
+  auto kfrag_of = [&](auto buf, int nb, int ks) -> i32x4 {
+    return *reinterpret_cast<const i32x4 *>(smem + SM::OFF_K + (int)buf * SM::K_BYTES + 32 * nb * SM::KSTR + kq[ks]);
+  };
   // S^T block nb (32 keys) of the tile held in K buffer `buf`, for this wave's 32 queries
   auto qk_block = [&](int buf, int nb, i32x16 &s) __attribute__((always_inline)) {
-    const unsigned char *ks_ = smem + SM::OFF_K + buf * SM::K_BYTES;
 #pragma unroll
     for (int v = 0; v < 16; ++v) s[v] = 0;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const i32x4 kf =
-          *reinterpret_cast<const i32x4 *>(ks_ + (32 * nb + lr) * SM::KSTR + (((2 * ks + g) ^ k_swz) << 4));
-      s = mfma_i8(kf, qf[ks], s);
-    }
+    for (int ks = 0; ks < KS; ++ks) s = mfma_i8(kfrag_of(buf, nb, ks), qf[ks], s);
   };
 
   f32x16 oacc[DB];
@@ -220,19 +275,16 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   auto prep = [&](int cbuf, int nb, const i32x16 &s, float (&u)[16], int j0, auto masked_tag)
                   __attribute__((always_inline)) -> float {
     constexpr bool MASKED = decltype(masked_tag)::value;
-    const unsigned char *cb = smem + SM::OFF_C + cbuf * SM::C_BYTES;
-    const float *skp = reinterpret_cast<const float *>(cb);
-    const u32x2 *dgp = reinterpret_cast<const u32x2 *>(cb + FWD_BN * 4);
     f32x16 f;
 #pragma unroll
     for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
-    const u32x2 corr_k = dgp[2 * (32 * nb + lr) + g];
-    f = mfma_16b_k8<T>(corr_k, corr_q, f);
+    // no bias here (this path also serves the rows that may not have one): the slot that meets the constant is zero
+    f = mfma_16b_k8<T>(corr_of(cbuf, nb), u32x2{corr_q[0], 0u}, f);
     float mt = -INFINITY;
 #pragma unroll
     for (int aa = 0; aa < 4; ++aa) {
       const int jl = 32 * nb + 8 * aa + 4 * g;
-      const f32x4 sk4 = *reinterpret_cast<const f32x4 *>(skp + jl);
+      const f32x4 sk4 = sk_of(cbuf, nb, aa);
 #pragma unroll
       for (int bb = 0; bb < 4; ++bb) {
         float uu = f[4 * aa + bb] * sk4[bb];
@@ -277,13 +329,13 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
     }
     // keys 32nb + 16hh + 4g + {0..3} and those + 8: the order in which pf holds the probabilities.
     // The reads are issued behind the compiler's back (see lds_read_tr16_async) and waited for below.
-    const unsigned vbase = lds_addr(smem + SM::OFF_V) + vbuf * SM::V_BYTES + (32 * nb + 4 * g) * SM::VSTR;
+    const unsigned voff = vbuf * SM::V_BYTES + 32 * nb * SM::VSTR;
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh) {
       u32x2 vr[2 * DB];
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const unsigned ad = vbase + hh * (16 * SM::VSTR) + (v_off ^ (64 * db));
+        const unsigned ad = vq[db] + voff + hh * (16 * SM::VSTR);
         vr[2 * db] = lds_read_tr16_async<0>(ad);
         vr[2 * db + 1] = lds_read_tr16_async<8 * SM::VSTR>(ad);
       }
@@ -304,7 +356,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
 
   // ---- prologue: K(0), K(1) (with their constants) and V(0) resident
   load_k(0, 0);
-  load_v(0);
+  load_v(0, 0);
   store_k(0);
   if (ntiles > 1) {
     load_k(1, 1);
@@ -313,42 +365,53 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   dma_wait();
   __syncthreads();
 
-  // tiles [0, t_hot) contain no masked score for this wave (wave-uniform)
+  // tiles [0, t_hot) contain no masked score for this wave (wave-uniform); a wave whose queries may not use
+  // biased accumulators takes the masked loop for every tile
   int t_hot = a.Nk / FWD_BN;
   if (CAUSAL) t_hot = min(t_hot, (q_first + coff + 1) / FWD_BN);
   t_hot = min(t_hot, ntiles);
+  if (!bias_ok) t_hot = 0;
 
-  int kb_cur = 0, kb_nxt = 1, kb_free = 2;   // K/constant buffers of tile t, t+1, and the one to refill
+  int kb_cur = 0, kb_nxt = 1, kb_free = 2;   // buffers of tile t, t+1, and the one to refill: t % 3, (t+1) % 3, (t+2) % 3
   int t = 0;
   if (t_hot > 0) {
     // ---- pipelined loop over unmasked tiles, one straight-line body per 32-key block b:
-    //   exp2/pack and P.V of block b | INT8 product of block b+1 | convert/correct/scale of b+1,
+    //   exp2/pack and P.V of block b | correction + INT8 product of block b+1 | unbias/scale of b+1,
     // with every LDS operand requested a phase (or a body) before the MFMA that consumes it and every MFMA
-    // result read a phase after the MFMA was issued (the chain convert -> correction MFMA -> scale is spread
-    // over the two P.V phases).  The
+    // result read a phase after the MFMA was issued.  The
     // phases are fenced so that the requests stay where they are; inside a phase MFMA and VALU
     // instructions are independent and interleave.  A wave raises its issue priority for the phases that
     // hold MFMAs and drops it for the ones that wait and request, so that of the two waves of a SIMD the
     // one that can feed the matrix pipe goes first (2 % at the non-causal sizes, nothing at the causal ones).
-    // Carried between bodies: u = prepared scores of block b, kf = K fragments of block b+1.
+    // Carried between bodies: u = prepared scores of block b, kf / ck = K fragments and correction operand of block b+1.
     float u[16];
     i32x4 kf[KS];
-    auto k_frags = [&](int buf, int nb) {
-      const unsigned char *ks_ = smem + SM::OFF_K + buf * SM::K_BYTES;
+    u32x2 ck;
+    // buffer indices are either ints or integral constants (the loop unrolled over three tiles): with constants
+    // every address below is a loop-invariant register plus an immediate
+    auto k_frags = [&](auto buf, int nb) {
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        kf[ks] = *reinterpret_cast<const i32x4 *>(ks_ + (32 * nb + lr) * SM::KSTR + (((2 * ks + g) ^ k_swz) << 4));
+      for (int ks = 0; ks < KS; ++ks) kf[ks] = kfrag_of(buf, nb, ks);
+      ck = corr_of(buf, nb);
     };
     // V fragments of keys 32nb + 16hh + 4g + {0..3} and those + 8 (the order in which pf holds the
     // probabilities), requested without the compiler's knowledge: pair every call with lds_wait_async
-    auto v_frags = [&](int vbuf, auto nb_tag, auto hh_tag, u32x2 (&vr)[2 * DB]) {
+    auto v_frags = [&](auto vbuf, auto nb_tag, auto hh_tag, u32x2 (&vr)[2 * DB]) {
       constexpr int ROW0 = (32 * decltype(nb_tag)::value + 16 * decltype(hh_tag)::value) * SM::VSTR;
-      const unsigned base = lds_addr(smem + SM::OFF_V) + vbuf * SM::V_BYTES + 4 * g * SM::VSTR;
+      if constexpr (is_static_int<decltype(vbuf)>::value && 2 * SM::V_BYTES + 56 * SM::VSTR < 65536) {
+        constexpr int IMM = decltype(vbuf)::value * SM::V_BYTES + ROW0;
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const unsigned ad = base + (v_off ^ (64 * db));
-        vr[2 * db] = lds_read_tr16_async<ROW0>(ad);
-        vr[2 * db + 1] = lds_read_tr16_async<ROW0 + 8 * SM::VSTR>(ad);
+        for (int db = 0; db < DB; ++db) {
+          vr[2 * db] = lds_read_tr16_async<IMM>(vq[db]);
+          vr[2 * db + 1] = lds_read_tr16_async<IMM + 8 * SM::VSTR>(vq[db]);
+        }
+      } else {
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const unsigned ad = vq[db] + (int)vbuf * SM::V_BYTES;
+          vr[2 * db] = lds_read_tr16_async<ROW0>(ad);
+          vr[2 * db + 1] = lds_read_tr16_async<ROW0 + 8 * SM::VSTR>(ad);
+        }
       }
     };
     // lnew = l_run + the 8 probabilities (the running sum continues in a second register, so that l_run is still
@@ -373,7 +436,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
     // through many terms is not brought down by the maximum of the current block alone).
     constexpr float SUM_LIMIT = 0x1p60f;
     auto check_half = [&](int hh, u32x4 &pf, float &lnew) {
-      if (__builtin_amdgcn_ballot_w64(!(lnew <= SUM_LIMIT)) != 0) {
+      if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(lnew <= SUM_LIMIT)) != 0, 0)) {
         float mt = m_ref + __log2f(fmaxf(l_run, 1.0f)) / a_i;
 #pragma unroll
         for (int v = 8 * hh; v < 16; ++v) mt = fmaxf(mt, u[v]);   // first half: the whole block
@@ -382,52 +445,58 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
       }
       l_run = lnew;
     };
-    // one body: V block (vbuf, nb); scores of the next block from kf; its constants in (cbuf, cnb);
-    // then kf is refilled from K block (kbuf, knb).
+    // one body: P.V of V block (vbuf, NB) with the scores in u; scores of the next block from kf / ck, scaled with the
+    // key scales of block (cbuf, CNB); then kf / ck are refilled from block (kbuf, KNB).
     // `copy(i)`, i = 0..2, is called between phases: the steady loop issues chunks of the next
     // tiles' copies there, so that the memory pipe sees a few requests at a time instead of a burst per tile
-    auto body = [&](int vbuf, auto nb_tag, int cbuf, int cnb, int kbuf, int knb, auto &&copy)
+    auto body = [&](auto vbuf, auto nb_tag, auto cbuf, auto cnb_tag, auto kbuf, auto knb_tag, auto &&copy)
                     __attribute__((always_inline)) {
       static_assert(DB == 8 || DB == 4 || DB == 2, "fragment arrays are sized for head_dim 256, 128 or 64");
+      constexpr int CNB = decltype(cnb_tag)::value, KNB = decltype(knb_tag)::value;
       u32x2 vr0[2 * DB], vr1[2 * DB];
       u32x4 pf0, pf1;
-      i32x16 s;
       const auto NB = nb_tag;
       // The K fragments were requested a body ago.  The compiler's counted wait for them must come HERE,
       // before the V requests it does not know of: in front of the INT8 MFMAs it would cover those too
       // (LDS returns in order) and the matrix pipe would idle for a full LDS round trip per block.
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(kf[ks]));
-      if (!QK_ONLY) v_frags(vbuf, NB, std::integral_constant<int, 0>{}, vr0);
+      asm volatile("" : "+v"(ck));
+      if (!QK_ONLY) v_frags(vbuf, NB, ic<0>{}, vr0);
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(1);
-      // INT8 product of block b+1 under the exponentials of the first 16 keys of block b
+      // zero-point correction plus bias first (exact: an integer in [2^23, 2^24)), then the INT8 product of block b+1
+      // accumulated onto its bit pattern, under the exponentials of the first 16 keys of block b
+      i32x16 s;
+      {
+        f32x16 y;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) s[v] = 0;
+        for (int v = 0; v < 16; ++v) y[v] = 0.f;
+        y = mfma_16b_k8<T>(ck, corr_q, y);
+        s = __builtin_bit_cast(i32x16, y);
+      }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) s = mfma_i8(kf[ks], qf[ks], s);
       float l0, l1;
       if (!QK_ONLY) exp_half(0, pf0, l0);
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(0);
-      copy(std::integral_constant<int, 0>{});
+      copy(ic<0>{});
       if (!QK_ONLY) {
         check_half(0, pf0, l0);
-        v_frags(vbuf, NB, std::integral_constant<int, 1>{}, vr1);
+        v_frags(vbuf, NB, ic<1>{}, vr1);
         lds_wait_async<(2 * DB < 15 ? 2 * DB : 15)>(vr0);   // the 2*DB requests just made may still be in flight (the counter holds 15)
       }
-      const unsigned char *cb = smem + SM::OFF_C + cbuf * SM::C_BYTES;
       f32x4 sk4[4];
 #pragma unroll
-      for (int aa = 0; aa < 4; ++aa)
-        sk4[aa] = *reinterpret_cast<const f32x4 *>(cb + (32 * cnb + 8 * aa + 4 * g) * 4);
-      const u32x2 corr_k = reinterpret_cast<const u32x2 *>(cb + FWD_BN * 4)[2 * (32 * cnb + lr) + g];
+      for (int aa = 0; aa < 4; ++aa) sk4[aa] = sk_of(cbuf, CNB, aa);
       __builtin_amdgcn_sched_barrier(0);
-      // P.V of the first 16 keys under the exponentials of the second 16 and the conversion of the next
-      // block's raw scores; their zero-point correction (one MFMA) goes last, so that its result has the
-      // whole next phase to arrive before the scaling reads it
+      // The MFMA that takes the bias out of the next block's scores goes first (the matrix pipe works in order: behind
+      // the four P.V products its result would arrive after the scaling wants it); then P.V of the first 16 keys
+      // under the exponentials of the second 16
       __builtin_amdgcn_s_setprio(1);
-      f32x16 f;
+      const f32x16 f = mfma_16b_k8<T>(unbias_a, corr_q, __builtin_bit_cast(f32x16, s));
+      __builtin_amdgcn_sched_barrier(0);
       if (!QK_ONLY) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
@@ -440,18 +509,14 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
         for (int v = 0; v < 16; ++v) sm = fmaxf(sm, u[v]);
         l_run = fmaxf(l_run, sm);
       }
-#pragma unroll
-      for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
-      __builtin_amdgcn_sched_barrier(0);
-      f = mfma_16b_k8<T>(corr_k, corr_q, f);
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(0);
       if (!QK_ONLY) {
         check_half(1, pf1, l1);
         lds_wait_async<0>(vr1);   // everything requested so far was requested a phase ago
       }
-      copy(std::integral_constant<int, 1>{});
-      k_frags(kbuf, knb);
+      copy(ic<1>{});
+      k_frags(kbuf, KNB);
       __builtin_amdgcn_sched_barrier(0);
       // P.V of the second 16 keys under the scaling of the next block's scores
       __builtin_amdgcn_s_setprio(1);
@@ -467,7 +532,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
         for (int bb = 0; bb < 4; ++bb) u[4 * aa + bb] = f[4 * aa + bb] * sk4[aa][bb];
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(0);
-      copy(std::integral_constant<int, 2>{});
+      copy(ic<2>{});
     };
 
     {   // block 0 prepared, fragments of block 1 in flight
@@ -480,38 +545,49 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
       k_frags(0, 1);
     }
     auto no_copy = [](auto) {};
-    // steady state: K(t+2) and V(t+1) are full tiles; their chunks (K first, then V) go out two at a
-    // time between the phases of the tile's first body, so that the last of them has the whole second body
-    // to land before the wait at the end of the tile (2 % at the causal headline size against one chunk
-    // per phase over both bodies; all six at once, or three and three, are slower again)
-    for (; t < t_hot && t + 2 < ntiles && (t + 3) * FWD_BN <= a.Nk; ++t) {
-      load_kc(t + 2);
+    // steady state, three tiles per trip (tile t in buffers t % 3 = B0): K(t+2) and V(t+1) are full tiles; their
+    // chunks (K first, then V) go out two at a time between the phases of the tile's first body, so that the last
+    // of them has the whole second body to land before the wait at the end of the tile (2 % at the causal headline
+    // size against one chunk per phase over both bodies; all six at once, or three and three, are slower again)
+    auto steady_tile = [&](auto b0_tag, int tt) __attribute__((always_inline)) {
+      constexpr int B0 = decltype(b0_tag)::value, B1 = (B0 + 1) % 3, B2 = (B0 + 2) % 3;
+      load_kc(tt + 2);
       const rsrc_t rs_k =
-          make_rsrc(reinterpret_cast<const unsigned char *>(kc_bh) + (int64_t)(t + 2) * FWD_BN * a.skn, 0x7fffffffu);
+          make_rsrc(reinterpret_cast<const unsigned char *>(kc_bh) + (int64_t)(tt + 2) * FWD_BN * a.skn, 0x7fffffffu);
       const rsrc_t rs_v = make_rsrc(
-          reinterpret_cast<const unsigned char *>(v_bh) + (int64_t)(t + 1) * FWD_BN * a.svn * (int64_t)sizeof(T), 0x7fffffffu);
-      unsigned char *kd = smem + SM::OFF_K + kb_free * SM::K_BYTES, *vd = smem + SM::OFF_V + ((t + 1) & 1) * SM::V_BYTES;
+          reinterpret_cast<const unsigned char *>(v_bh) + (int64_t)(tt + 1) * FWD_BN * a.svn * (int64_t)sizeof(T), 0x7fffffffu);
+      unsigned char *kd = smem + SM::OFF_K + B2 * SM::K_BYTES, *vd = smem + SM::OFF_V + B1 * SM::V_BYTES;
       constexpr int KCH = decltype(cp_k)::N, VCH = decltype(cp_v)::N;
       auto chunk = [&](int i) {   // i is a compile-time constant at every call site
-        if (i < KCH) cp_k.issue_one(rs_k, kd, wave_u, tid, i);
-        else if (i < KCH + VCH) cp_v.issue_one(rs_v, vd, wave_u, tid, i - KCH);
+        if (i < KCH) cp_k.issue_one(rs_k, kd, wave_u, i);
+        else if (i < KCH + VCH) cp_v.issue_one(rs_v, vd, wave_u, i - KCH);
       };
       constexpr int PER = (KCH + VCH + 2) / 3;   // chunks per slot: 2 at head_dim 128, 4 at 256
-      body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, [&](auto i) {
+      body(ic<B0>{}, ic<0>{}, ic<B0>{}, ic<1>{}, ic<B1>{}, ic<0>{}, [&](auto i) {
 #pragma unroll
         for (int c = 0; c < PER; ++c) chunk(PER * decltype(i)::value + c);
       });
-      body(t & 1, std::integral_constant<int, 1>{}, kb_nxt, 0, kb_nxt, 1, no_copy);
-      store_k(kb_free);
-      const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
+      body(ic<B0>{}, ic<1>{}, ic<B1>{}, ic<0>{}, ic<B1>{}, ic<1>{}, no_copy);
+      store_k(B2);
       dma_wait();
       __syncthreads();
+    };
+    {
+      // tiles [0, t_steady) are unmasked for this wave, and their copies (two tiles ahead) are full tiles
+      const int t_steady = min(t_hot, min(ntiles - 2, a.Nk / FWD_BN - 2));
+      for (; t + 3 <= t_steady; t += 3) {
+        steady_tile(ic<0>{}, t);
+        steady_tile(ic<1>{}, t + 1);
+        steady_tile(ic<2>{}, t + 2);
+      }
     }
+    // the rest of the unmasked tiles (at most two of the steady kind, then the ones whose copies are ragged or
+    // missing), with run-time buffer indices; t % 3 == 0 here
     for (; t < t_hot; ++t) {
       if (t + 2 < ntiles) load_k(t + 2, kb_free);
-      if (t + 1 < ntiles) load_v(t + 1);
-      body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, no_copy);
-      body(t & 1, std::integral_constant<int, 1>{}, kb_nxt, 0, kb_nxt, 1, no_copy);
+      if (t + 1 < ntiles) load_v(t + 1, kb_nxt);
+      body(kb_cur, ic<0>{}, kb_cur, ic<1>{}, kb_nxt, ic<0>{}, no_copy);
+      body(kb_cur, ic<1>{}, kb_nxt, ic<0>{}, kb_nxt, ic<1>{}, no_copy);
       if (t + 2 < ntiles) store_k(kb_free);
       const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
       dma_wait();
@@ -526,10 +602,10 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
     if (!QK_ONLY && CAUSAL && D <= 128 && t < ntiles && coff % 32 == 0 && t == (q_first + coff + 1) / FWD_BN &&
         (t + 1) * FWD_BN <= a.Nk) {
       if (t + 2 < ntiles) load_k(t + 2, kb_free);
-      if (t + 1 < ntiles) load_v(t + 1);
+      if (t + 1 < ntiles) load_v(t + 1, kb_nxt);
       const int j0 = t * FWD_BN;
       const int nb_d = (q_first + coff - j0) / 32;   // 0 or 1, wave-uniform: the block that holds the diagonal
-      if (nb_d == 1) body(t & 1, std::integral_constant<int, 0>{}, kb_cur, 1, kb_nxt, 0, no_copy);
+      if (nb_d == 1) body(kb_cur, ic<0>{}, kb_cur, ic<1>{}, kb_nxt, ic<0>{}, no_copy);
       float mt = -INFINITY;
 #pragma unroll
       for (int aa = 0; aa < 4; ++aa)
@@ -540,7 +616,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
           mt = fmaxf(mt, u[4 * aa + bb]);
         }
       rescale_if_needed(max_across_halves(mt));
-      exp_pv(t & 1, nb_d, u);
+      exp_pv(kb_cur, nb_d, u);
       if (t + 2 < ntiles) store_k(kb_free);
       const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
       dma_wait();
@@ -551,7 +627,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   // ---- masked tiles (diagonal, ragged end): one block at a time, nothing carried between blocks
   for (; t < ntiles; ++t) {
     if (t + 2 < ntiles) load_k(t + 2, kb_free);
-    if (t + 1 < ntiles) load_v(t + 1);
+    if (t + 1 < ntiles) load_v(t + 1, kb_nxt);
     const int j0 = t * FWD_BN;
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
@@ -561,7 +637,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
       float u[16];
       qk_block(kb_cur, nb, s);
       rescale_if_needed(prep(kb_cur, nb, s, u, j0, std::true_type{}));
-      exp_pv(t & 1, nb, u);
+      exp_pv(kb_cur, nb, u);
     }
     if (t + 2 < ntiles) store_k(kb_free);
     const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
@@ -578,8 +654,8 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   const float inv = 1.0f / l_tot;
   // O leaves as whole rows through LDS (all tile buffers are free after the last barrier; every wave takes 32 * 2D
   // bytes at the start of the K area)
-  static_assert(FWD_WAVES * 32 * 2 * D <= SM::OFF_V + 2 * SM::V_BYTES, "output staging fits the tile buffers");
-  store_tile_rows<T, D>(oacc, inv, smem + wave * (32 * 2 * D), o_bh, a.son, m0 + wave * 32, a.Nq, lane);
+  static_assert(SM::OFF_K + FWD_WAVES * 32 * 2 * D <= SM::TOTAL, "output staging fits the tile buffers");
+  store_tile_rows<T, D>(oacc, inv, smem + SM::OFF_K + wave * (32 * 2 * D), o_bh, a.son, m0 + wave * 32, a.Nq, lane);
   if (qi < a.Nq && g == 0) a.lse[tq0 + qi] = (a_i * m_ref + __log2f(l_tot)) * kLn2;
 }
 

@@ -31,15 +31,20 @@ template <int D> struct FwdSmem {
   static constexpr int VSTR = 2 * D;             // bytes per V row (dense, quarters swizzled: SwzQuad<2D>)
   static constexpr int K_BYTES = FWD_BN * KSTR;
   static constexpr int V_BYTES = FWD_BN * VSTR;
-  static constexpr int C_BYTES = FWD_BN * 4 + FWD_BN * 16;  // key scale; correction operands (per key and k-group a pair and a zero dword)
-  static constexpr int OFF_K = 0;                     // 3 buffers
-  static constexpr int OFF_V = 3 * K_BYTES;           // 2 buffers
-  static constexpr int OFF_C = OFF_V + 2 * V_BYTES;   // 3 buffers
-  static constexpr int TOTAL = OFF_C + 3 * C_BYTES;
-  // head_dim 128: two workgroups share a CU's 160 KB (2 waves per SIMD of up to 256 registers); head_dim 64: three
-  // (the loop fits the 168 registers of three waves per SIMD without spills: 10 % faster than two); head_dim 256:
-  // 114 KB, one workgroup, each wave has the SIMD's whole register file (the 128 O accumulators live in AccVGPRs)
-  static constexpr int WG_PER_CU = 3 * TOTAL <= 160 * 1024 ? 3 : 2 * TOTAL <= 160 * 1024 ? 2 : 1;
+  static constexpr int C_BYTES = FWD_BN * 4 + FWD_BN * 16;  // key scale; correction operands (per key and k-group two dwords)
+  // Tile t lives in buffer t % 3 of each of the three rings, so that a loop unrolled over three tiles addresses
+  // all of them with immediate offsets
+  static constexpr int NBUF = 3;
+  static constexpr int OFF_C = 0;                     // the small ring first: its reads keep 16-bit immediate offsets
+  static constexpr int OFF_K = OFF_C + NBUF * C_BYTES;
+  static constexpr int OFF_V = OFF_K + NBUF * K_BYTES;
+  static constexpr int TOTAL = OFF_V + NBUF * V_BYTES;
+  static_assert(OFF_K % 256 == 0 && OFF_V % 256 == 0, "tile buffers start on a bank line");
+  // head_dim 128: two workgroups per CU (2 waves per SIMD of up to 256 registers; 76 KB of LDS each); head_dim 64:
+  // three (the loop fits the 168 registers of three waves per SIMD: 10 % faster than two); head_dim 256: 148 KB,
+  // one workgroup, each wave has the SIMD's whole register file (the 128 O accumulators live in AccVGPRs)
+  static constexpr int WG_PER_CU = D <= 64 ? 3 : D <= 128 ? 2 : 1;
+  static_assert(WG_PER_CU * TOTAL <= 160 * 1024, "the workgroups of a CU share 160 KB of LDS");
 };
 
 // integer n in [-32768, 32767] -> (128*floor(n/128), n mod 128) as a packed pair of 16-bit floats
