@@ -282,6 +282,27 @@ template <int OFF> __device__ __forceinline__ u32x2 lds_read_tr16_async(unsigned
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
   return r;
 }
+// The same for plain 16-byte and 8-byte reads (a loop that times every LDS request itself issues all of them this way)
+template <int OFF> __device__ __forceinline__ u32x4 lds_read_b128_async(unsigned addr) {
+  u32x4 r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+template <int OFF> __device__ __forceinline__ u32x2 lds_read_b64_async(unsigned addr) {
+  u32x2 r;
+  asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+// wait until at most N LDS operations of this wave are outstanding; the values named are tied behind the wait
+template <typename A> __device__ __forceinline__ void lds_tie(A &a) { asm volatile("" : "+v"(a)); }
+template <typename A, int K> __device__ __forceinline__ void lds_tie(A (&a)[K]) {
+#pragma unroll
+  for (int i = 0; i < K; ++i) asm volatile("" : "+v"(a[i]));
+}
+template <int N, typename... A> __device__ __forceinline__ void lds_wait_for(A &...a) {
+  asm volatile("s_waitcnt lgkmcnt(%0)" : : "n"(N) : "memory");
+  (lds_tie(a), ...);
+}
 template <int N> __device__ __forceinline__ void lds_wait_async(u32x2 (&r)[8]) {
   asm volatile("s_waitcnt lgkmcnt(%8)"
                : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7])

@@ -81,6 +81,10 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   typedef FwdSmem<D> SM;
   constexpr int KS = D / 32;   // int8 k-steps of 32
   constexpr int DB = D / 32;   // 32-row blocks of O^T
+  // Biased accumulators (see the head of the file) up to head_dim 128.  At head_dim 256 a wave is alone on its SIMD
+  // and the longer dependent chain (correction -> 8 INT8 products -> unbias) is not hidden by anybody: measured 35 %
+  // slower there than converting explicitly.
+  constexpr bool BIAS = D <= 128;
   __shared__ __attribute__((aligned(256))) unsigned char smem[SM::TOTAL];
 
   // ---- block -> (batch*head, query block); consecutive ids of one XCD share a head's K/V in its L2
@@ -370,7 +374,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   int t_hot = a.Nk / FWD_BN;
   if (CAUSAL) t_hot = min(t_hot, (q_first + coff + 1) / FWD_BN);
   t_hot = min(t_hot, ntiles);
-  if (!bias_ok) t_hot = 0;
+  if (BIAS && !bias_ok) t_hot = 0;
 
   int kb_cur = 0, kb_nxt = 1, kb_free = 2;   // buffers of tile t, t+1, and the one to refill: t % 3, (t+1) % 3, (t+2) % 3
   int t = 0;
@@ -468,12 +472,15 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
       // zero-point correction plus bias first (exact: an integer in [2^23, 2^24)), then the INT8 product of block b+1
       // accumulated onto its bit pattern, under the exponentials of the first 16 keys of block b
       i32x16 s;
-      {
+      if constexpr (BIAS) {
         f32x16 y;
 #pragma unroll
         for (int v = 0; v < 16; ++v) y[v] = 0.f;
         y = mfma_16b_k8<T>(ck, corr_q, y);
         s = __builtin_bit_cast(i32x16, y);
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] = 0;
       }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) s = mfma_i8(kf[ks], qf[ks], s);
@@ -495,8 +502,11 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
       // the four P.V products its result would arrive after the scaling wants it); then P.V of the first 16 keys
       // under the exponentials of the second 16
       __builtin_amdgcn_s_setprio(1);
-      const f32x16 f = mfma_16b_k8<T>(unbias_a, corr_q, __builtin_bit_cast(f32x16, s));
-      __builtin_amdgcn_sched_barrier(0);
+      f32x16 f;
+      if constexpr (BIAS) {
+        f = mfma_16b_k8<T>(unbias_a, corr_q, __builtin_bit_cast(f32x16, s));
+        __builtin_amdgcn_sched_barrier(0);
+      }
       if (!QK_ONLY) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
@@ -508,6 +518,13 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
 #pragma unroll
         for (int v = 0; v < 16; ++v) sm = fmaxf(sm, u[v]);
         l_run = fmaxf(l_run, sm);
+      }
+      if constexpr (!BIAS) {
+        // explicit conversion, then the correction product (its query side without the bias slot)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) f[v] = (float)s[v];
+        __builtin_amdgcn_sched_barrier(0);
+        f = mfma_16b_k8<T>(ck, u32x2{corr_q[0], 0u}, f);
       }
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(0);
@@ -545,44 +562,53 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
       k_frags(0, 1);
     }
     auto no_copy = [](auto) {};
-    // steady state, three tiles per trip (tile t in buffers t % 3 = B0): K(t+2) and V(t+1) are full tiles; their
+    // steady state (tile t in buffers t % 3 = b0, b1 and b2 the next two): K(t+2) and V(t+1) are full tiles; their
     // chunks (K first, then V) go out two at a time between the phases of the tile's first body, so that the last
     // of them has the whole second body to land before the wait at the end of the tile (2 % at the causal headline
     // size against one chunk per phase over both bodies; all six at once, or three and three, are slower again)
-    auto steady_tile = [&](auto b0_tag, int tt) __attribute__((always_inline)) {
-      constexpr int B0 = decltype(b0_tag)::value, B1 = (B0 + 1) % 3, B2 = (B0 + 2) % 3;
+    auto steady_tile = [&](auto b0, auto b1, auto b2, int tt) __attribute__((always_inline)) {
       load_kc(tt + 2);
       const rsrc_t rs_k =
           make_rsrc(reinterpret_cast<const unsigned char *>(kc_bh) + (int64_t)(tt + 2) * FWD_BN * a.skn, 0x7fffffffu);
       const rsrc_t rs_v = make_rsrc(
           reinterpret_cast<const unsigned char *>(v_bh) + (int64_t)(tt + 1) * FWD_BN * a.svn * (int64_t)sizeof(T), 0x7fffffffu);
-      unsigned char *kd = smem + SM::OFF_K + B2 * SM::K_BYTES, *vd = smem + SM::OFF_V + B1 * SM::V_BYTES;
+      unsigned char *kd = smem + SM::OFF_K + (int)b2 * SM::K_BYTES, *vd = smem + SM::OFF_V + (int)b1 * SM::V_BYTES;
       constexpr int KCH = decltype(cp_k)::N, VCH = decltype(cp_v)::N;
       auto chunk = [&](int i) {   // i is a compile-time constant at every call site
         if (i < KCH) cp_k.issue_one(rs_k, kd, wave_u, i);
         else if (i < KCH + VCH) cp_v.issue_one(rs_v, vd, wave_u, i - KCH);
       };
       constexpr int PER = (KCH + VCH + 2) / 3;   // chunks per slot: 2 at head_dim 128, 4 at 256
-      body(ic<B0>{}, ic<0>{}, ic<B0>{}, ic<1>{}, ic<B1>{}, ic<0>{}, [&](auto i) {
+      body(b0, ic<0>{}, b0, ic<1>{}, b1, ic<0>{}, [&](auto i) {
 #pragma unroll
         for (int c = 0; c < PER; ++c) chunk(PER * decltype(i)::value + c);
       });
-      body(ic<B0>{}, ic<1>{}, ic<B1>{}, ic<0>{}, ic<B1>{}, ic<1>{}, no_copy);
-      store_k(B2);
+      body(b0, ic<1>{}, b1, ic<0>{}, b1, ic<1>{}, no_copy);
+      store_k((int)b2);
       dma_wait();
       __syncthreads();
     };
     {
       // tiles [0, t_steady) are unmasked for this wave, and their copies (two tiles ahead) are full tiles
       const int t_steady = min(t_hot, min(ntiles - 2, a.Nk / FWD_BN - 2));
-      for (; t + 3 <= t_steady; t += 3) {
-        steady_tile(ic<0>{}, t);
-        steady_tile(ic<1>{}, t + 1);
-        steady_tile(ic<2>{}, t + 2);
+      if constexpr (D <= 128 && !QK_ONLY) {
+        // three tiles per trip with constant buffer indices
+        for (; t + 3 <= t_steady; t += 3) {
+          steady_tile(ic<0>{}, ic<1>{}, ic<2>{}, t);
+          steady_tile(ic<1>{}, ic<2>{}, ic<0>{}, t + 1);
+          steady_tile(ic<2>{}, ic<0>{}, ic<1>{}, t + 2);
+        }
+      } else {
+        // head_dim 256: one tile per trip (the unrolled loop is three times 1 400 instructions there, and the V
+        // offsets exceed the immediate field anyway)
+        for (; t < t_steady; ++t) {
+          steady_tile(kb_cur, kb_nxt, kb_free, t);
+          const int tmp = kb_cur; kb_cur = kb_nxt; kb_nxt = kb_free; kb_free = tmp;
+        }
       }
     }
     // the rest of the unmasked tiles (at most two of the steady kind, then the ones whose copies are ragged or
-    // missing), with run-time buffer indices; t % 3 == 0 here
+    // missing), with run-time buffer indices (kb_cur == t % 3 here)
     for (; t < t_hot; ++t) {
       if (t + 2 < ntiles) load_k(t + 2, kb_free);
       if (t + 1 < ntiles) load_v(t + 1, kb_nxt);
