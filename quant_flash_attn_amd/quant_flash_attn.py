@@ -352,12 +352,13 @@ class QuantFlashAttention(torch.autograd.Function):
 def _normalised_dout(grad_output: torch.Tensor, kv_scale: torch.Tensor):
     """(dO * 2^k as float16, 2^-k as a one-element float32 tensor) for the binary16 backward kernels.
 
-    k puts the largest |dO| at 2^8 when the key scales are of the usual size (2^-5 for values of order
-    one) and higher when they are smaller, since the smallest operand the kernels form carries the
-    key scale as a factor; dO * 2^k itself stays below 2^14.  Everything is computed on the device."""
+    k puts the largest |dO| * 2^k * (largest key scale) at 8: 2^8 for |dO| when the key scales are of the usual size
+    (2^-5 for values of order one), higher when they are smaller and lower when they are larger, since the operands
+    the kernels form carry the key scale as a factor (ds * scale_j must neither sink into binary16's subnormals nor
+    leave its range); dO * 2^k itself stays below 2^14.  Everything is computed on the device."""
     do32 = grad_output.to(torch.float32)
     amax = do32.abs().amax().clamp_min(1e-30)
-    smax = kv_scale.to(torch.float32).abs().amax().clamp(1e-30, 2.0 ** -5)
+    smax = kv_scale.to(torch.float32).abs().amax().clamp_min(1e-30)
     k = torch.minimum(torch.floor(torch.log2(8.0 / (amax * smax))), torch.floor(torch.log2(16384.0 / amax)))
     k = k.clamp_(-100.0, 100.0)
     return (do32 * torch.exp2(k)).to(torch.float16), torch.exp2(-k)

@@ -28,17 +28,23 @@ def max_abs(a: torch.Tensor, b: torch.Tensor) -> float:
 # (fp64 evaluation of the same formulas), which is why `want` takes the saved O.
 MAX_ABS_TOL = 2e-2
 COS_TOL = 0.999
+# cosine bar for a reference whose RMS lies below the absolute bar (see assert_close): 0.99 still rejects a result that
+# is zero, has the wrong sign or misses a tenth of the reference in any direction
+SMALL_COS_TOL = 0.99
 REL_TOL = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}
 
 
-def assert_close(name, got, want, max_abs_tol=MAX_ABS_TOL, cos_tol=COS_TOL, scaled=False, rel=None, spread=None):
+def assert_close(name, got, want, max_abs_tol=MAX_ABS_TOL, cos_tol=COS_TOL, scaled=False, rel=None, spread=None,
+                 small_cos_tol=SMALL_COS_TOL):
     """scaled=False: max|got - want| <= max_abs_tol.  scaled=True (gradients, and outputs that are not of order
-    one): |got - want| <= max_abs_tol + rel * (|want| + spread) element-wise, rel from got's dtype unless given."""
+    one): |got - want| <= max_abs_tol + rel * (|want| + spread) element-wise; rel is the rounding step of got's dtype
+    and must be given when got is not a 16-bit tensor (there is no default to fall back on)."""
     assert torch.isfinite(got.float()).all(), f"{name}: non-finite values"
     cs = cosine(got, want)
     err = (got.double() - want.double()).abs()
     if scaled:
-        r = REL_TOL.get(got.dtype, 2.0 ** -7) if rel is None else rel
+        assert rel is not None or got.dtype in REL_TOL, f"{name}: pass rel= for a {got.dtype} result"
+        r = REL_TOL[got.dtype] if rel is None else rel
         size = want.double().abs() if spread is None else want.double().abs() + spread.double()
         excess = err - (max_abs_tol + r * size)
         worst = int(excess.argmax())
@@ -48,13 +54,17 @@ def assert_close(name, got, want, max_abs_tol=MAX_ABS_TOL, cos_tol=COS_TOL, scal
     else:
         ok = bool(err.max() <= max_abs_tol)
         detail = f"max-abs {float(err.max()):.3e} (tol {max_abs_tol:.3e})"
-    # A reference whose typical element lies below the absolute bar has no direction to compare at the contract's
-    # resolution: nearly one-hot softmax rows leave dQ as the small difference of large terms (two dominant keys
+    # A reference whose typical element lies below the absolute bar is compared at a coarser angle, never at none:
+    # nearly one-hot softmax rows leave dQ as the small difference of large terms (two dominant keys
     # give dQ_i = sm * dS_i1 * (k_1 - k_2) with the keys' common part cancelled), where the 16-bit operands'
-    # rounding is a few percent of the result while every element is 25 times inside the element-wise bound.
-    if float(want.double().pow(2).mean().sqrt()) < max_abs_tol:
-        cos_tol = -1.0
-    assert ok and cs >= cos_tol, f"{name}: {detail}, cosine {cs:.6f} (tol {cos_tol})"
+    # rounding is a few percent of the result while every element is 25 times inside the element-wise bound
+    # (measured: 0.9978); a result of zero, which the absolute bar alone would let through there, has cosine 0.
+    rms = float(want.double().pow(2).mean().sqrt())
+    if rms < 1e-3 * max_abs_tol:
+        cos_tol = -1.0   # a reference that is zero at the bar's resolution has no direction; the absolute bar holds got to zero
+    elif rms < max_abs_tol:
+        cos_tol = min(cos_tol, small_cos_tol)
+    assert ok and cs >= cos_tol, f"{name}: {detail}, cosine {cs:.6f} (tol {cos_tol}), RMS of the reference {rms:.3e}"
     return float(err.max()), cs
 
 
@@ -65,8 +75,8 @@ def rounded_output_floor(qh, kh, v, do, o_ref, lse_ref, out_dtype, causal, sm):
     rounding, and no kernel can be closer to the exact gradients than these values are."""
     Nq, Nk = qh.shape[-2], kh.shape[-2]
     s = (qh @ kh.transpose(-1, -2)) * sm
-    if causal:
-        s = s.masked_fill(torch.arange(Nk)[None, :] > torch.arange(Nq)[:, None], float("-inf"))
+    if causal:   # aligned to the last key, as in the kernels and the oracle
+        s = s.masked_fill(torch.arange(Nk)[None, :] > torch.arange(Nq)[:, None] + (Nk - Nq), float("-inf"))
     p = torch.exp(s - lse_ref.double()[..., None])
     delta = (o_ref.to(out_dtype).double() * do.double()).sum(-1, keepdim=True)
     ds = p * (do.double() @ v.double().transpose(-1, -2) - delta)
