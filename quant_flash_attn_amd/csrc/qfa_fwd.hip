@@ -50,8 +50,8 @@
 // block become one MFMA.  The two range conditions (|corr| and |S| below 2^22, intermediate sums of the first
 // MFMA below 2^24 in any order) are checked per query in the prologue from quantities the wave has anyway
 // (|zq|, |rq - D zq| and sum_d |qc_d - zq|, bounded against the worst key); a wave with a query that could leave
-// the window -- rows pinned at one end of the code range -- takes the masked loop, which converts explicitly, for
-// all its tiles.
+// the window -- rows pinned at one end of the code range, e.g. all-positive rows -- runs the instance of the same
+// loop that converts explicitly (2 % slower).
 //
 // Head dimensions 64, 128 and 256 are instances of the same code: three, two and one workgroup per CU.
 //
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   // Biased accumulators (see the head of the file) up to head_dim 128.  At head_dim 256 a wave is alone on its SIMD
   // and the longer dependent chain (correction -> 8 INT8 products -> unbias) is not hidden by anybody: measured 35 %
   // slower there than converting explicitly.
-  constexpr bool BIAS = D <= 128;
+  constexpr bool BIAS_POSSIBLE = D <= 128;
   __shared__ __attribute__((aligned(256))) unsigned char smem[SM::TOTAL];
 
   // ---- block -> (batch*head, query block); consecutive ids of one XCD share a head's K/V in its L2
@@ -154,8 +154,10 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   //   |terms of the first MFMA| <= |zq| (128 D + 127) + 128 (|c| + 2 * 2^SH) =: tq   (|rk digit sum| <= 128 D + 127, |zk| <= 128)
   //   |S| <= 255 * sum_d |qc_d - zq| =: 255 mq
   // and both must stay below 2^22.
-  bool bias_ok;
-  {
+  // (at head_dim 64 both bounds hold for every possible row: 255 * 64 * 255 and 128 * 8319 + 128 * 16576 are below 2^22)
+  constexpr bool BIAS_ALWAYS = D <= 64;
+  bool bias_ok = true;
+  if constexpr (!BIAS_ALWAYS && BIAS_POSSIBLE) {
     const unsigned zb = ((unsigned)(zq_i + 128) & 0xffu) * 0x01010101u;
     unsigned mq = 0;
 #pragma unroll
@@ -369,16 +371,15 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
   dma_wait();
   __syncthreads();
 
-  // tiles [0, t_hot) contain no masked score for this wave (wave-uniform); a wave whose queries may not use
-  // biased accumulators takes the masked loop for every tile
+  // tiles [0, t_hot) contain no masked score for this wave (wave-uniform)
   int t_hot = a.Nk / FWD_BN;
   if (CAUSAL) t_hot = min(t_hot, (q_first + coff + 1) / FWD_BN);
   t_hot = min(t_hot, ntiles);
-  if (BIAS && !bias_ok) t_hot = 0;
 
   int kb_cur = 0, kb_nxt = 1, kb_free = 2;   // buffers of tile t, t+1, and the one to refill: t % 3, (t+1) % 3, (t+2) % 3
   int t = 0;
-  if (t_hot > 0) {
+  auto pipelined = [&](auto bias_tag) __attribute__((always_inline)) {
+    constexpr bool BIAS = decltype(bias_tag)::value;
     // ---- pipelined loop over unmasked tiles, one straight-line body per 32-key block b:
     //   exp2/pack and P.V of block b | correction + INT8 product of block b+1 | unbias/scale of b+1,
     // with every LDS operand requested a phase (or a body) before the MFMA that consumes it and every MFMA
@@ -648,6 +649,18 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
       dma_wait();
       __syncthreads();
       ++t;
+    }
+  };
+  // Two instances of the pipelined part: with biased accumulators for the waves whose queries allow them, with the
+  // explicit conversion for the others (rows pinned at an end of the code range; all-positive rows are the common case)
+  if (t_hot > 0) {
+    if constexpr (BIAS_ALWAYS) {
+      pipelined(std::true_type{});
+    } else if constexpr (BIAS_POSSIBLE) {
+      if (bias_ok) pipelined(std::true_type{});
+      else pipelined(std::false_type{});
+    } else {
+      pipelined(std::false_type{});
     }
   }
   // ---- masked tiles (diagonal, ragged end): one block at a time, nothing carried between blocks

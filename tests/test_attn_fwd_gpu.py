@@ -139,6 +139,49 @@ def test_constant_rows_at_the_clamps_give_exact_integer_scores(qfa, D, causal):
     assert float(rel.max()) < 1e-6
 
 
+def _may_use_biased_accumulators(qq, D):
+    """The kernel's per-query test (head_dim <= 128), restated: every term of the zero-point correction and the
+    integer score itself must stay below 2^22 against the worst key."""
+    codes = qq.codes.cpu().long()
+    zq = qq.zero_point.cpu().long().reshape(codes.shape[:-1])
+    c = qq.rowsum.cpu().long().reshape(zq.shape) - D * zq
+    mq = (codes - zq[..., None]).abs().sum(-1)
+    tq = zq.abs() * (128 * D + 127) + 128 * (c.abs() + 2 * 128)
+    return (255 * mq < 2 ** 22) & (tq < 2 ** 22)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("mixed", [False, True])
+def test_rows_that_may_not_use_biased_accumulators(qfa, D, causal, mixed):
+    """Query rows that sit at one end of their range (all elements in [0.5, 1]: zero point -128, every code +127)
+    fail the bound under which the pipelined loop may accumulate the INT8 product onto a biased fp32 bit pattern:
+    their waves run the instance of the loop that converts explicitly.  Long enough for the unrolled steady loop;
+    `mixed` puts rows of either kind into one workgroup (the choice is per wave of 32 queries)."""
+    B, H, N = 1, 2, 704
+    g = torch.Generator().manual_seed(11 * D + 2 * causal + mixed)
+    q = torch.randn((B, H, N, D), generator=g)
+    k = torch.randn((B, H, N, D), generator=g)
+    v = torch.randn((B, H, N, D), generator=g).to(torch.bfloat16)
+    pinned = 0.5 + 0.5 * torch.rand((B, H, N, D), generator=g)
+    if mixed:
+        q[:, :, 32:64] = pinned[:, :, 32:64]
+        q[:, :, 300:420] = -pinned[:, :, 300:420]
+    else:
+        q = pinned
+    q, k = q.to(torch.bfloat16), k.to(torch.bfloat16)
+    sm = 1.0 / math.sqrt(D)
+    qq, kq, o, lse = _run(qfa, q, k, v, causal, sm)
+    ok = _may_use_biased_accumulators(qq, D)
+    if D == 64:   # no row can leave the window at this width: the kernel does not even look
+        assert ok.all()
+    else:
+        assert not ok[:, :, 32:64].any() and (mixed == bool(ok[:, :, 64:96].all()))
+    o_ref, lse_ref = _oracle_fwd(qq, kq, v, causal, sm)
+    assert_close("O", o.cpu(), o_ref)
+    assert max_abs(lse.cpu(), lse_ref) < 2.0 ** -8
+
+
 def test_fp32_plumbing_configuration(qfa):
     """B1 H4 N256 D64 fp32 q,k,v, seed 0, non-causal, through the autograd entry point."""
     torch.manual_seed(0)
