@@ -152,8 +152,7 @@ def main():
     # ---- the timed region: K steps of (quantize Q, quantize K, forward), wall clock, with HIP
     # events around every attention launch for the kernel's own duration
     def step(evs=None):
-        qq = qfa.quantize_for_attention(q)
-        kq = qfa.quantize_for_attention(k)
+        qq, kq = qfa.quantize_pair_for_attention(q, k)   # both tensors in one launch, as quant_flash_attn_qkv does
         if evs is not None:
             evs[0].record()
         o, lse = qfa.attn_fwd_quantized(qq, kq, v, causal, sm)

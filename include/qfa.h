@@ -68,6 +68,19 @@ int qfa_quant_per_token(const void *x, int x_dtype, int8_t *codes, float *scale_
                         void *stream);
 
 /*
+ * qfa_quant_per_token for TWO tensors of one element type and head dimension in one launch: the queries and the keys
+ * of an attention call (tensor 0: [B,H,N0,D], tensor 1: [B,H,N1,D]).  Replaces the two launches of
+ * _asymmetric_quant_kernel (asymmetric_quant.py:132-147) that quantizing q and k costs; same arithmetic, same
+ * outputs per tensor (codes, fp32 scale, zero point, optional row sum; no 16-bit copy of the scale), one launch
+ * ramp and one tail instead of two.  Strides in elements: x per tensor (b, h, n), codes per tensor (b, h, n).
+ */
+int qfa_quant_per_token_pair(const void *x0, const void *x1, int x_dtype, int8_t *codes0, int8_t *codes1,
+                             float *scale0, float *scale1, int8_t *zp0, int8_t *zp1, int32_t *rowsum0, int32_t *rowsum1,
+                             int64_t B, int64_t H, int64_t N0, int64_t N1, int D, int64_t sx0b, int64_t sx0h,
+                             int64_t sx0n, int64_t sx1b, int64_t sx1h, int64_t sx1n, int64_t sc0b, int64_t sc0h,
+                             int64_t sc0n, int64_t sc1b, int64_t sc1h, int64_t sc1n, void *stream);
+
+/*
  * out = (codes - zp) * scale, per token (asymmetric_quant.py:158-160, and the in-kernel
  * dequantization quant_flash_attn.py:65).  scale_dtype is the element type of `scale`
  * (QFA_F32 / QFA_F16 / QFA_BF16); out has out_dtype and strides sob,soh,son.

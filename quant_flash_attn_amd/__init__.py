@@ -12,7 +12,7 @@ libqfa.so (C ABI in include/qfa.h):
 GPU only: a CPU tensor or a missing libqfa.so raises; there is no fallback implementation.
 """
 from .asymmetric_quant import (QuantizedTokens, asymmetric_quant_per_token, code_rowsum, dequantize_per_token,
-                               quantize_for_attention)
+                               quantize_for_attention, quantize_pair_for_attention)
 from .quant_flash_attn import (QuantFlashAttention, QuantFlashAttnQKV, attn_bwd_quantized, attn_fwd_quantized,
                                attn_bwd_shared_kv, attn_fwd_shared_kv,
                                QuantFlashAttnQuantizedKV, quant_flash_attn, quant_flash_attn_qkv,
@@ -20,6 +20,7 @@ from .quant_flash_attn import (QuantFlashAttention, QuantFlashAttnQKV, attn_bwd_
 
 __all__ = [
     "QuantizedTokens", "asymmetric_quant_per_token", "code_rowsum", "dequantize_per_token", "quantize_for_attention",
+    "quantize_pair_for_attention",
     "QuantFlashAttention", "QuantFlashAttnQKV", "QuantFlashAttnQuantizedKV", "quant_flash_attn", "quant_flash_attn_qkv",
     "quant_flash_attn_quantized_kv",
     "attn_fwd_quantized", "attn_bwd_quantized", "attn_fwd_shared_kv", "attn_bwd_shared_kv",

@@ -25,6 +25,7 @@ _SIGNATURES = {
     "qfa_version": (c_int, []),
     "qfa_last_error": (ctypes.c_char_p, []),
     "qfa_quant_per_token": (c_int, [_P, _I, _P, _P, _P, _I, _P, _P, _L, _L, _L, _I] + [_L] * 6 + [_P]),
+    "qfa_quant_per_token_pair": (c_int, [_P, _P, _I] + [_P] * 8 + [_L, _L, _L, _L, _I] + [_L] * 12 + [_P]),
     "qfa_dequant_per_token": (c_int, [_P, _P, _I, _P, _P, _I, _L, _L, _L, _I] + [_L] * 6 + [_P]),
     "qfa_code_rowsum": (c_int, [_P, _P, _L, _L, _L, _I, _L, _L, _L, _P]),
     "qfa_attn_fwd": (c_int, [_P] * 11 + [_I, _L, _L, _L, _L, _I] + [_L] * 12 + [_F, _I, _P]),

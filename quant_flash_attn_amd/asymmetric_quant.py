@@ -78,6 +78,31 @@ def quantize_for_attention(x: torch.Tensor) -> QuantizedTokens:
     return QuantizedTokens(codes, scale32, zp, rowsum)
 
 
+def quantize_pair_for_attention(x0: torch.Tensor, x1: torch.Tensor) -> Tuple[QuantizedTokens, QuantizedTokens]:
+    """quantize_for_attention of two tensors (the queries and the keys of an attention call: same batch, heads,
+    head dimension and element type, any two lengths) in ONE launch; bit-identical to two separate calls."""
+    x0, x1 = _check_input(x0), _check_input(x1)
+    if x0.shape[:2] != x1.shape[:2] or x0.shape[3] != x1.shape[3] or x0.dtype != x1.dtype or x0.device != x1.device:
+        return quantize_for_attention(x0), quantize_for_attention(x1)
+    B, H, _, D = x0.shape
+    out = []
+    for x in (x0, x1):
+        N = x.shape[2]
+        out.append((torch.empty((B, H, N, D), dtype=torch.int8, device=x.device),
+                    torch.empty((B, H, N, 1), dtype=torch.float32, device=x.device),
+                    torch.empty((B, H, N, 1), dtype=torch.int8, device=x.device),
+                    torch.empty((B, H, N, 1), dtype=torch.int32, device=x.device)))
+    (c0, s0, z0, r0), (c1, s1, z1, r1) = out
+    with torch.cuda.device(x0.device):
+        code = _lib.lib().qfa_quant_per_token_pair(
+            x0.data_ptr(), x1.data_ptr(), _lib.DTYPE_CODE[x0.dtype], c0.data_ptr(), c1.data_ptr(), s0.data_ptr(),
+            s1.data_ptr(), z0.data_ptr(), z1.data_ptr(), r0.data_ptr(), r1.data_ptr(), B, H, x0.shape[2], x1.shape[2], D,
+            x0.stride(0), x0.stride(1), x0.stride(2), x1.stride(0), x1.stride(1), x1.stride(2),
+            c0.stride(0), c0.stride(1), c0.stride(2), c1.stride(0), c1.stride(1), c1.stride(2), _lib.stream_of(x0))
+    _lib.check(code, "qfa_quant_per_token_pair")
+    return QuantizedTokens(c0, s0, z0, r0), QuantizedTokens(c1, s1, z1, r1)
+
+
 def dequantize_per_token(codes: torch.Tensor, scale: torch.Tensor, zero_point: torch.Tensor,
                          dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """(codes - zero_point) * scale per token (the reference's dequantize_per_token_torch,

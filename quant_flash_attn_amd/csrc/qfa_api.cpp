@@ -67,6 +67,33 @@ int qfa_quant_per_token(const void *x, int x_dtype, int8_t *codes, float *scale_
                       scb, sch, scn, (hipStream_t)stream);
 }
 
+int qfa_quant_per_token_pair(const void *x0, const void *x1, int x_dtype, int8_t *codes0, int8_t *codes1,
+                             float *scale0, float *scale1, int8_t *zp0, int8_t *zp1, int32_t *rowsum0, int32_t *rowsum1,
+                             int64_t B, int64_t H, int64_t N0, int64_t N1, int D, int64_t sx0b, int64_t sx0h,
+                             int64_t sx0n, int64_t sx1b, int64_t sx1h, int64_t sx1n, int64_t sc0b, int64_t sc0h,
+                             int64_t sc0n, int64_t sc1b, int64_t sc1h, int64_t sc1n, void *stream) {
+  const void *const x[2] = {x0, x1};
+  int8_t *const codes[2] = {codes0, codes1};
+  float *const scale[2] = {scale0, scale1};
+  int8_t *const zp[2] = {zp0, zp1};
+  int32_t *const rowsum[2] = {rowsum0, rowsum1};
+  const int64_t N[2] = {N0, N1};
+  const int64_t sx[2][3] = {{sx0b, sx0h, sx0n}, {sx1b, sx1h, sx1n}}, sc[2][3] = {{sc0b, sc0h, sc0n}, {sc1b, sc1h, sc1n}};
+  if (!is_float_dtype(x_dtype)) return set_error(QFA_EINVAL, "quant_pair: x_dtype %d is not QFA_F32/F16/BF16", x_dtype);
+  if (B <= 0 || H <= 0 || N0 <= 0 || N1 <= 0) return set_error(QFA_EINVAL, "quant_pair: B, H, N0, N1 must be positive");
+  if (D < 8 || D > 256 || D % 8 != 0)
+    return set_error(QFA_EUNSUPPORTED, "quant_pair: head_dim %d is not a multiple of 8 between 8 and 256", D);
+  for (int i = 0; i < 2; ++i) {
+    if (!x[i] || !codes[i] || !scale[i] || !zp[i]) return set_error(QFA_EINVAL, "quant_pair: null x/codes/scale/zp pointer");
+    if (!aligned16(x[i]) || !aligned8(codes[i])) return set_error(QFA_EINVAL, "quant_pair: x must be 16-byte, codes 8-byte aligned");
+    if (!strides_ok(sx[i][0], sx[i][1], sx[i][2], D, elem_size(x_dtype)))
+      return set_error(QFA_EINVAL, "quant_pair: x strides must be positive multiples of 16 bytes, token stride >= D");
+    if (sc[i][0] <= 0 || sc[i][1] <= 0 || sc[i][2] < D || sc[i][0] % 8 != 0 || sc[i][1] % 8 != 0 || sc[i][2] % 8 != 0)
+      return set_error(QFA_EINVAL, "quant_pair: codes strides must be positive multiples of 8 bytes, token stride >= D");
+  }
+  return launch_quant_pair(x, x_dtype, codes, scale, zp, rowsum, B, H, N, D, sx, sc, (hipStream_t)stream);
+}
+
 int qfa_dequant_per_token(const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp, void *out,
                           int out_dtype, int64_t B, int64_t H, int64_t N, int D, int64_t scb, int64_t sch,
                           int64_t scn, int64_t sob, int64_t soh, int64_t son, void *stream) {

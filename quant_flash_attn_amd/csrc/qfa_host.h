@@ -16,6 +16,10 @@ int check_launch(const char *what);
 int launch_quant(const void *x, int x_dtype, int8_t *codes, float *scale, void *scale_lp, int scale_lp_dtype,
                  int8_t *zp, int32_t *rowsum, int64_t B, int64_t H, int64_t N, int D, int64_t sxb, int64_t sxh,
                  int64_t sxn, int64_t scb, int64_t sch, int64_t scn, hipStream_t st);
+// the same for two tensors of one element type and head dimension in one launch (no 16-bit scale copy)
+int launch_quant_pair(const void *const x[2], int x_dtype, int8_t *const codes[2], float *const scale[2],
+                      int8_t *const zp[2], int32_t *const rowsum[2], int64_t B, int64_t H, const int64_t N[2], int D,
+                      const int64_t sx[2][3], const int64_t sc[2][3], hipStream_t st);
 int launch_rowsum(const int8_t *codes, int32_t *rowsum, int64_t B, int64_t H, int64_t N, int D, int64_t scb,
                   int64_t sch, int64_t scn, hipStream_t st);
 int launch_dequant(const int8_t *codes, const void *scale, int scale_dtype, const int8_t *zp, void *out,

@@ -104,15 +104,16 @@ struct QuantArgs {
 
 // One block = 256 threads = U passes over 256/(DP/8) tokens of one (b,h) slice.  DP = the head dimension
 // rounded up to a power of two; PARTIAL: the head dimension is smaller than DP.
-template <typename T, int DP, int U, bool PARTIAL> __global__ __launch_bounds__(256) void quant_kernel(QuantArgs a) {
+template <typename T, int DP, int U, bool PARTIAL>
+__device__ __forceinline__ void quant_block(const QuantArgs &a, unsigned block) {
   constexpr int LPT = DP / 8;         // lanes per token
   constexpr int TPP = 256 / LPT;      // tokens per pass
   const int tid = threadIdx.x;
   const int sub = tid % LPT;
   const bool lane_used = !PARTIAL || sub * 8 < a.D;
   const int sub_ld = lane_used ? sub : 0;   // idle lanes duplicate the token's first eight elements
-  const int64_t bh = blockIdx.x / a.chunks_per_bh;
-  const int64_t chunk = blockIdx.x % a.chunks_per_bh;
+  const int64_t bh = block / a.chunks_per_bh;
+  const int64_t chunk = block % a.chunks_per_bh;
   const int64_t b = bh / a.H, h = bh % a.H;
   const int64_t n0 = chunk * (int64_t)(TPP * U) + tid / LPT;
   const T *xb = reinterpret_cast<const T *>(a.x) + b * a.sxb + h * a.sxh;
@@ -201,6 +202,20 @@ template <typename T, int DP, int U, bool PARTIAL> __global__ __launch_bounds__(
   }
 }
 
+template <typename T, int DP, int U, bool PARTIAL> __global__ __launch_bounds__(256) void quant_kernel(QuantArgs a) {
+  quant_block<T, DP, U, PARTIAL>(a, blockIdx.x);
+}
+// Two tensors of one element type and head dimension in one launch (the queries and the keys of an attention call):
+// the first blocks0 workgroups take tensor 0, the others tensor 1.  One launch ramp and one tail instead of two.
+struct QuantPairArgs {
+  QuantArgs t[2];
+  unsigned blocks0;
+};
+template <typename T, int DP, int U, bool PARTIAL> __global__ __launch_bounds__(256) void quant_pair_kernel(QuantPairArgs p) {
+  if (blockIdx.x < p.blocks0) quant_block<T, DP, U, PARTIAL>(p.t[0], blockIdx.x);
+  else quant_block<T, DP, U, PARTIAL>(p.t[1], blockIdx.x - p.blocks0);
+}
+
 template <typename T, int DP> static int launch_quant_d(const QuantArgs &a0, int64_t BH, hipStream_t st) {
   constexpr int U = 4;
   constexpr int TOK = (256 / (DP / 8)) * U;
@@ -238,6 +253,51 @@ int launch_quant(const void *x, int x_dtype, int8_t *codes, float *scale, void *
     case QFA_BF16: return launch_quant_t<__bf16>(a, B * H, st);
   }
   return set_error(QFA_EINVAL, "quant: bad x_dtype");
+}
+
+template <typename T, int DP> static int launch_quant_pair_d(QuantPairArgs p, int64_t BH, hipStream_t st) {
+  constexpr int U = 4;
+  constexpr int TOK = (256 / (DP / 8)) * U;
+  int64_t blocks[2];
+  for (int i = 0; i < 2; ++i) {
+    const int64_t chunks = (p.t[i].N + TOK - 1) / TOK;
+    p.t[i].chunks_per_bh = (int)chunks;
+    blocks[i] = chunks * BH;
+  }
+  if (blocks[0] + blocks[1] > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "quant_pair: too many tokens for one launch");
+  p.blocks0 = (unsigned)blocks[0];
+  const dim3 grid((unsigned)(blocks[0] + blocks[1])), block(256);
+  if (p.t[0].D == DP) quant_pair_kernel<T, DP, U, false><<<grid, block, 0, st>>>(p);
+  else quant_pair_kernel<T, DP, U, true><<<grid, block, 0, st>>>(p);
+  return check_launch("qfa_quant_per_token_pair");
+}
+template <typename T> static int launch_quant_pair_t(const QuantPairArgs &p, int64_t BH, hipStream_t st) {
+  switch (padded_head_dim(p.t[0].D)) {
+    case 32: return launch_quant_pair_d<T, 32>(p, BH, st);
+    case 64: return launch_quant_pair_d<T, 64>(p, BH, st);
+    case 128: return launch_quant_pair_d<T, 128>(p, BH, st);
+  }
+  return launch_quant_pair_d<T, 256>(p, BH, st);
+}
+
+int launch_quant_pair(const void *const x[2], int x_dtype, int8_t *const codes[2], float *const scale[2],
+                      int8_t *const zp[2], int32_t *const rowsum[2], int64_t B, int64_t H, const int64_t N[2], int D,
+                      const int64_t sx[2][3], const int64_t sc[2][3], hipStream_t st) {
+  QuantPairArgs p;
+  for (int i = 0; i < 2; ++i) {
+    QuantArgs &a = p.t[i];
+    a.x = x[i]; a.codes = codes[i]; a.scale = scale[i]; a.scale_lp = nullptr; a.zp = zp[i]; a.rowsum = rowsum[i];
+    a.N = N[i]; a.H = H; a.sxb = sx[i][0]; a.sxh = sx[i][1]; a.sxn = sx[i][2];
+    a.scb = sc[i][0]; a.sch = sc[i][1]; a.scn = sc[i][2];
+    a.chunks_per_bh = 0; a.scale_lp_dtype = 0; a.D = D;
+  }
+  p.blocks0 = 0;
+  switch (x_dtype) {
+    case QFA_F32: return launch_quant_pair_t<float>(p, B * H, st);
+    case QFA_F16: return launch_quant_pair_t<_Float16>(p, B * H, st);
+    case QFA_BF16: return launch_quant_pair_t<__bf16>(p, B * H, st);
+  }
+  return set_error(QFA_EINVAL, "quant_pair: bad x_dtype");
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -23,7 +23,8 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from .asymmetric_quant import QuantizedTokens, code_rowsum, dequantize_per_token, quantize_for_attention
+from .asymmetric_quant import (QuantizedTokens, code_rowsum, dequantize_per_token, quantize_for_attention,
+                               quantize_pair_for_attention)
 
 _IO_DTYPES = (torch.bfloat16, torch.float16)
 
@@ -235,8 +236,7 @@ class QuantFlashAttnQKV(torch.autograd.Function):
             raise ValueError("q, k, v must be 4-D (Batch, Heads, Seq, Head_Dim)")
         if q.shape[-1] != k.shape[-1] or k.shape != v.shape or q.shape[:2] != k.shape[:2]:
             raise ValueError(f"shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
-        qq = quantize_for_attention(q)
-        kq = quantize_for_attention(k)
+        qq, kq = quantize_pair_for_attention(q, k)   # one launch for both
         v16 = v.to(_io_dtype(v))
         o, lse = attn_fwd_quantized(qq, kq, v16, causal, sm_scale)
         ctx.save_for_backward(*qq, *kq, v16, o, lse)

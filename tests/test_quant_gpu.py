@@ -134,3 +134,18 @@ def test_outputs_fully_written_and_deterministic(qfa):
     b = qfa.quantize_for_attention(xg)
     for s, t in zip(a, b):
         assert torch.equal(s, t)
+
+
+@pytest.mark.parametrize("D,dtype", [(128, torch.bfloat16), (64, torch.float16), (40, torch.float32), (256, torch.bfloat16)])
+def test_pair_launch_is_bit_identical_to_two_launches(qfa, D, dtype):
+    """quantize_pair_for_attention (queries and keys in one launch, qfa_quant_per_token_pair) against two calls of
+    quantize_for_attention: every output tensor bit for bit, with different lengths and a strided second tensor."""
+    g = torch.Generator().manual_seed(D)
+    q = (torch.randn((2, 3, 333, D), generator=g) * 1.7 + 0.3).to(dtype).to(DEV)
+    k_store = (torch.randn((2, 1029, 3, D), generator=g) - 0.5).to(dtype).to(DEV)   # [B,N,H,D] storage
+    k = k_store.permute(0, 2, 1, 3)
+    a0, a1 = qfa.quantize_pair_for_attention(q, k)
+    b0, b1 = qfa.quantize_for_attention(q), qfa.quantize_for_attention(k)
+    for got, want in ((a0, b0), (a1, b1)):
+        for x, y in zip(got, want):
+            assert x.shape == y.shape and x.dtype == y.dtype and torch.equal(x, y)
