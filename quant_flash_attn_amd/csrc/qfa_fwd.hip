@@ -70,9 +70,9 @@ template <typename X> struct is_static_int : std::false_type {};
 template <int V> struct is_static_int<std::integral_constant<int, V>> : std::true_type {};
 template <int V> using ic = std::integral_constant<int, V>;
 
-// QK_ONLY is the measurement variant of the same kernel: identical loads, INT8 product, zero-point
-// correction, scaling and running maximum, with the exponentials and the P.V product compiled out
-// (it writes the scaled row maximum where the LSE would go and leaves O untouched).  It exists to
+// QK_ONLY is the measurement variant of the same kernel: identical K and constant loads, INT8 product, zero-point
+// correction, scaling and a maximum over the scores, with the V copies, the exponentials and the P.V product compiled
+// out (it writes the scaled row maximum where the LSE would go and leaves O untouched).  It exists to
 // time the QK^T stage by itself against the INT8 MFMA peak.
 template <typename T, int D, bool CAUSAL, bool QK_ONLY = false, int NW = FWD_WAVES>
 __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(FwdArgs a) {
@@ -227,6 +227,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
     }
   };
   auto load_v = [&](int t, int buf) {
+    if (QK_ONLY) return;   // the QK^T-stage variant multiplies nothing by V
     const int j0 = t * FWD_BN;
     unsigned char *dst = smem + SM::OFF_V + buf * SM::V_BYTES;
     const int64_t vstride = a.svn * (int64_t)sizeof(T);
@@ -577,7 +578,7 @@ __global__ __launch_bounds__(64 * NW, FwdSmem<D>::WG_PER_CU) void fwd_kernel(Fwd
       constexpr int KCH = decltype(cp_k)::N, VCH = decltype(cp_v)::N;
       auto chunk = [&](int i) {   // i is a compile-time constant at every call site
         if (i < KCH) cp_k.issue_one(rs_k, kd, wave_u, i);
-        else if (i < KCH + VCH) cp_v.issue_one(rs_v, vd, wave_u, i - KCH);
+        else if (i < KCH + VCH && !QK_ONLY) cp_v.issue_one(rs_v, vd, wave_u, i - KCH);
       };
       constexpr int PER = (KCH + VCH + 2) / 3;   // chunks per slot: 2 at head_dim 128, 4 at 256
       body(b0, ic<0>{}, b0, ic<1>{}, b1, ic<0>{}, [&](auto i) {
