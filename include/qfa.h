@@ -222,6 +222,14 @@ int qfa_bench_qk_stage(const int8_t *qc, const float *sq, const int8_t *zq, cons
                        int64_t sob, int64_t soh, int64_t son, float sm_scale, int causal, void *stream);
 
 /*
+ * out[i] = a[i] + b[i] for two dense 16-bit tensors of n elements (n a multiple of 8, pointers 16-byte aligned;
+ * out may be a or b), added in fp32 and rounded once.  The merged gradient dkv = dv + dk that _bwd_kernel_quantized
+ * stores for its shared K = V tensor (quant_flash_attn.py:161), for callers that obtained dK and dV from
+ * qfa_attn_bwd (query blocks too long for qfa_attn_bwd_shared_kv).
+ */
+int qfa_sum_grads(const void *a, const void *b, void *out, int dtype, int64_t n, void *stream);
+
+/*
  * delta[b,h,n] = sum_d O[b,h,n,d] * dO[b,h,n,d], accumulated in fp32.
  * Replaces the launch of _bwd_preprocess_kernel (quant_flash_attn.py:87-101, :217-223).
  * qfa_attn_bwd computes delta inside its own staging pass; this entry point is for callers that

@@ -295,6 +295,14 @@ int qfa_bwd_delta(const void *o, const void *dout, float *delta, int io_dtype, i
   return launch_delta(o, dout, delta, io_dtype, B, H, N, D, sob, soh, son, sdb, sdh, sdn, (hipStream_t)stream);
 }
 
+int qfa_sum_grads(const void *a, const void *b, void *out, int dtype, int64_t n, void *stream) {
+  if (!a || !b || !out) return set_error(QFA_EINVAL, "sum_grads: null pointer argument");
+  if (dtype != QFA_BF16 && dtype != QFA_F16) return set_error(QFA_EINVAL, "sum_grads: dtype must be QFA_BF16 or QFA_F16");
+  if (n <= 0 || n % 8 != 0) return set_error(QFA_EINVAL, "sum_grads: the element count must be a positive multiple of 8");
+  if (!aligned16(a) || !aligned16(b) || !aligned16(out)) return set_error(QFA_EINVAL, "sum_grads: pointers must be 16-byte aligned");
+  return launch_sum16(a, b, out, dtype, n, (hipStream_t)stream);
+}
+
 int64_t qfa_attn_bwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D) {
   if (B <= 0 || H <= 0 || Nq <= 0 || Nk <= 0 || (D != 64 && D != 128 && D != 256)) return 0;
   return bwd_workspace_bytes(B, H, Nq, Nk, D);

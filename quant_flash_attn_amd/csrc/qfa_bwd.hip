@@ -63,6 +63,28 @@ template <typename T, int D> __global__ __launch_bounds__(256) void delta_kernel
   if (n < a.N && sub == 0) a.delta[bh * a.N + n] = s;
 }
 
+// out = a + b for two 16-bit tensors of the same dense shape, added in fp32 and rounded once: dKV = dK + dV of the
+// shared K = V contract (quant_flash_attn.py:161) when the two gradients come from the INT8-score kernels.
+template <typename T> __global__ __launch_bounds__(256) void sum16_kernel(const T *a, const T *b, T *out, int64_t n8) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n8) return;
+  const u32x4 x = reinterpret_cast<const u32x4 *>(a)[i], y = reinterpret_cast<const u32x4 *>(b)[i];
+  u32x4 r;
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    r[e] = pack2<T>(lo_to_f32<T>(x[e]) + lo_to_f32<T>(y[e]), hi_to_f32<T>(x[e]) + hi_to_f32<T>(y[e]));
+  reinterpret_cast<u32x4 *>(out)[i] = r;
+}
+int launch_sum16(const void *a, const void *b, void *out, int dtype, int64_t n, hipStream_t st) {
+  const int64_t n8 = n / 8, blocks = (n8 + 255) / 256;
+  if (blocks > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "sum_grads: too many elements for one launch");
+  if (dtype == QFA_BF16)
+    sum16_kernel<__bf16><<<dim3((unsigned)blocks), dim3(256), 0, st>>>((const __bf16 *)a, (const __bf16 *)b, (__bf16 *)out, n8);
+  else
+    sum16_kernel<_Float16><<<dim3((unsigned)blocks), dim3(256), 0, st>>>((const _Float16 *)a, (const _Float16 *)b, (_Float16 *)out, n8);
+  return check_launch("qfa_sum_grads");
+}
+
 int launch_delta(const void *o, const void *dout, float *delta, int io_dtype, int64_t B, int64_t H, int64_t N, int D,
                  int64_t sob, int64_t soh, int64_t son, int64_t sdb, int64_t sdh, int64_t sdn, hipStream_t st) {
   DeltaArgs a;

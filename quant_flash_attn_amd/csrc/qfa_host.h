@@ -45,6 +45,7 @@ int launch_fwd(const AttnArgs &a, hipStream_t st, bool qk_only = false);
 int launch_delta(const void *o, const void *dout, float *delta, int io_dtype, int64_t B, int64_t H, int64_t N, int D,
                  int64_t sob, int64_t soh, int64_t son, int64_t sdb, int64_t sdh, int64_t sdn, hipStream_t st);
 int launch_bwd(const AttnArgs &a, hipStream_t st);
+int launch_sum16(const void *a, const void *b, void *out, int dtype, int64_t n, hipStream_t st);   // out = a + b, n % 8 == 0
 int64_t bwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D);
 
 // Shared-KV attention (K = V = one quantized tensor, Q in 16-bit float), after validation.

@@ -345,7 +345,12 @@ class QuantFlashAttention(torch.autograd.Function):
             qq, kq = QuantizedTokens(*t[0:4]), QuantizedTokens(*t[4:8])
             v16, o, lse = t[8], t[9], t[10]
         dq, dk, dv = attn_bwd_quantized(qq, kq, v16, o, grad_output.to(v16.dtype), lse, False, ctx.sm_scale)
-        dkv = dk.to(torch.float32).add_(dv).to(ctx.kv_dtype)      # :161 (dk already carries sm_scale)
+        # :161 (dk already carries sm_scale): one pass, added in fp32 and rounded once
+        dk, dv = dk.contiguous(), dv.contiguous()
+        with torch.cuda.device(dk.device):
+            _lib.check(_lib.lib().qfa_sum_grads(dk.data_ptr(), dv.data_ptr(), dk.data_ptr(), _lib.DTYPE_CODE[dk.dtype],
+                                                dk.numel(), _lib.stream_of(dk)), "qfa_sum_grads")
+        dkv = dk.to(ctx.kv_dtype)
         return dq.to(ctx.q_dtype), dkv, None, None
 
 
