@@ -222,6 +222,21 @@ int qfa_bench_qk_stage(const int8_t *qc, const float *sq, const int8_t *zq, cons
                        int64_t sob, int64_t soh, int64_t son, float sm_scale, int causal, void *stream);
 
 /*
+ * out = dout * 2^k as binary16 and back[0] = 2^-k, for a dense 16-bit dout of n elements (n a multiple of 8, dout and
+ * out 16-byte aligned) and the n_scale per-token scales of the shared K = V tensor (QFA_F32 or QFA_F16).
+ * qfa_attn_bwd_shared_kv computes in binary16 and forms sm_scale * p * (dP - delta) * scale_j as a matrix operand;
+ * dQ and dKV are linear in dO, so callers hand it this scaled dO and pass `back` as grad_scale.  k is the largest
+ * integer with  max|dout| * 2^k * max|scale| <= 8  and  max|dout| * 2^k <= 2^14  (within [-100, 100]), found on the
+ * device: two launches, no synchronisation, no atomics.  workspace: qfa_dout_normalise_workspace_bytes() bytes of
+ * device scratch (4-byte aligned), contents irrelevant before and after.  No counterpart in the reference, whose
+ * Triton kernel runs the same products in fp16 on dO as it comes (quant_flash_attn.py:130-161) and loses small
+ * gradients to fp16's subnormals.
+ */
+int64_t qfa_dout_normalise_workspace_bytes(void);
+int qfa_dout_normalise(const void *dout, int dout_dtype, int64_t n, const void *kv_scale, int scale_dtype, int64_t n_scale,
+                       void *workspace, void *out, float *back, void *stream);
+
+/*
  * out[i] = a[i] + b[i] for two dense 16-bit tensors of n elements (n a multiple of 8, pointers 16-byte aligned;
  * out may be a or b), added in fp32 and rounded once.  The merged gradient dkv = dv + dk that _bwd_kernel_quantized
  * stores for its shared K = V tensor (quant_flash_attn.py:161), for callers that obtained dK and dV from

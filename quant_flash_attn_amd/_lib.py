@@ -36,6 +36,8 @@ _SIGNATURES = {
                                + [_F, _P]),
     "qfa_bench_qk_stage": (c_int, [_P] * 11 + [_I, _L, _L, _L, _L, _I] + [_L] * 12 + [_F, _I, _P]),
     "qfa_sum_grads": (c_int, [_P, _P, _P, _I, _L, _P]),
+    "qfa_dout_normalise_workspace_bytes": (c_int64, []),
+    "qfa_dout_normalise": (c_int, [_P, _I, _L, _P, _I, _L, _P, _P, _P, _P]),
     "qfa_bwd_delta": (c_int, [_P, _P, _P, _I, _L, _L, _L, _I] + [_L] * 6 + [_P]),
     "qfa_attn_bwd_workspace_bytes": (c_int64, [_L, _L, _L, _L, _I]),
     "qfa_attn_bwd": (c_int, [_P] * 13 + [_L] + [_P] * 3 + [_I, _L, _L, _L, _L, _I] + [_L] * 24 + [_F, _I, _P]),

@@ -303,6 +303,20 @@ int qfa_sum_grads(const void *a, const void *b, void *out, int dtype, int64_t n,
   return launch_sum16(a, b, out, dtype, n, (hipStream_t)stream);
 }
 
+int64_t qfa_dout_normalise_workspace_bytes(void) { return dout_normalise_workspace_bytes(); }
+
+int qfa_dout_normalise(const void *dout, int dout_dtype, int64_t n, const void *kv_scale, int scale_dtype, int64_t n_scale,
+                       void *workspace, void *out, float *back, void *stream) {
+  if (!dout || !kv_scale || !workspace || !out || !back) return set_error(QFA_EINVAL, "dout_normalise: null pointer argument");
+  if (dout_dtype != QFA_BF16 && dout_dtype != QFA_F16) return set_error(QFA_EINVAL, "dout_normalise: dout_dtype must be QFA_BF16 or QFA_F16");
+  if (scale_dtype != QFA_F32 && scale_dtype != QFA_F16) return set_error(QFA_EINVAL, "dout_normalise: scale_dtype must be QFA_F32 or QFA_F16");
+  if (n <= 0 || n % 8 != 0) return set_error(QFA_EINVAL, "dout_normalise: the element count must be a positive multiple of 8");
+  if (n_scale <= 0) return set_error(QFA_EINVAL, "dout_normalise: n_scale must be positive");
+  if (!aligned16(dout) || !aligned16(out)) return set_error(QFA_EINVAL, "dout_normalise: dout and out must be 16-byte aligned");
+  return launch_dout_normalise(dout, dout_dtype, n, kv_scale, scale_dtype, n_scale, static_cast<float *>(workspace), out, back,
+                               (hipStream_t)stream);
+}
+
 int64_t qfa_attn_bwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, int D) {
   if (B <= 0 || H <= 0 || Nq <= 0 || Nk <= 0 || (D != 64 && D != 128 && D != 256)) return 0;
   return bwd_workspace_bytes(B, H, Nq, Nk, D);

@@ -66,6 +66,11 @@ int64_t skv_fwd_workspace_bytes(int64_t B, int64_t H, int64_t Nq, int64_t Nk, in
 // the same with the partial results of a split in the library's own static device array (a.workspace is ignored)
 int launch_skv_fwd_static(const SkvAttnArgs &a, hipStream_t st);
 int launch_skv_bwd(const SkvAttnArgs &a, hipStream_t st);        // io_dtype QFA_F16, Nq <= 32: one fused pass
+// dO * 2^k as binary16 plus 2^-k for the binary16 backward kernels (k from max|dO| and the largest key scale);
+// partials: dout_normalise_workspace_bytes() of scratch
+int64_t dout_normalise_workspace_bytes();
+int launch_dout_normalise(const void *dout, int dout_dtype, int64_t n, const void *scale, int scale_dtype, int64_t ns,
+                          float *partials, void *out, float *back, hipStream_t st);
 int launch_skv_bwd_long(const SkvAttnArgs &a, hipStream_t st);   // io_dtype QFA_F16, any Nq: dQ kernel + dKV kernel
 
 }  // namespace qfa

@@ -443,4 +443,93 @@ int launch_skv_bwd(const SkvAttnArgs &x, hipStream_t st) {
   return set_error(QFA_EUNSUPPORTED, "attn_bwd_shared_kv: head_dim must be 64, 128 or 256");
 }
 
+// ---- dO handed to the binary16 backward kernels: dO * 2^k as binary16, and 2^-k for the kernels to scale dQ and dKV
+// back with.  dQ and dKV are linear in dO, and what the kernels feed the matrix pipe is sm_scale * p * (dP - delta)
+// and that times the key's scale: k puts  max|dO| * 2^k * (largest key scale)  into (4, 8] and keeps
+// max|dO| * 2^k at or below 2^14, so that neither ordinary small gradients sink into binary16's subnormals nor large
+// key scales leave its range.  Two launches, no atomics: every block of the first writes its two partial maxima,
+// every block of the second reduces all of them again (a few KB out of the L2) before it scales its share.
+constexpr int NORM_BLOCKS = 512;   // blocks of the first launch = pairs of floats in the partials buffer
+
+template <typename T> __device__ __forceinline__ float max_abs8(const u32x4 w, float m) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) m = fmaxf(m, fmaxf(fabsf(lo_to_f32<T>(w[e])), fabsf(hi_to_f32<T>(w[e]))));
+  return m;
+}
+__device__ __forceinline__ float block_max_256(float m, float *red) {
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+  __syncthreads();
+  if (threadIdx.x % 64 == 0) red[threadIdx.x / 64] = m;
+  __syncthreads();
+  return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+// floor(log2(c / y)) for c = 2^ce and a positive normal y, exactly (no logarithm): y = m * 2^e with m in [1, 2)
+__device__ __forceinline__ int floor_log2_quot(int ce, float y) {
+  const unsigned b = __builtin_bit_cast(unsigned, y);
+  const int e = (int)((b >> 23) & 0xff) - 127;
+  return ce - e - ((b & 0x7fffffu) != 0 ? 1 : 0);
+}
+
+template <typename T, typename S>
+__global__ __launch_bounds__(256) void dout_max_kernel(const T *dout, int64_t n8, const S *scale, int64_t ns, float *partials) {
+  __shared__ float red[4];
+  float m = 0.f, ms = 0.f;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)NORM_BLOCKS * 256)
+    m = max_abs8<T>(reinterpret_cast<const u32x4 *>(dout)[i], m);
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < ns; i += (int64_t)NORM_BLOCKS * 256)
+    ms = fmaxf(ms, fabsf((float)scale[i]));
+  m = block_max_256(m, red);
+  ms = block_max_256(ms, red);
+  if (threadIdx.x == 0) {
+    partials[2 * blockIdx.x] = m;
+    partials[2 * blockIdx.x + 1] = ms;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void dout_scale_kernel(const T *dout, int64_t n8, const float *partials, _Float16 *out,
+                                                         float *back) {
+  __shared__ float red[4];
+  float m = 0.f, ms = 0.f;
+  for (int i = threadIdx.x; i < NORM_BLOCKS; i += 256) {
+    m = fmaxf(m, partials[2 * i]);
+    ms = fmaxf(ms, partials[2 * i + 1]);
+  }
+  m = fmaxf(block_max_256(m, red), 1e-30f);     // inf stays inf: k = -100 below
+  ms = fmaxf(block_max_256(ms, red), 1e-30f);
+  int k = min(floor_log2_quot(3, m * ms), floor_log2_quot(14, m));
+  k = max(-100, min(100, k));
+  const float f = __builtin_ldexpf(1.0f, k);
+  if (blockIdx.x == 0 && threadIdx.x == 0) back[0] = __builtin_ldexpf(1.0f, -k);
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n8) return;
+  const u32x4 w = reinterpret_cast<const u32x4 *>(dout)[i];
+  u32x4 r;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) r[e] = pack2<_Float16>(lo_to_f32<T>(w[e]) * f, hi_to_f32<T>(w[e]) * f);
+  reinterpret_cast<u32x4 *>(out)[i] = r;
+}
+
+template <typename T, typename S>
+static int launch_dout_normalise_ts(const void *dout, int64_t n, const void *scale, int64_t ns, float *partials,
+                                    void *out, float *back, hipStream_t st) {
+  const int64_t n8 = n / 8, blocks = (n8 + 255) / 256;
+  if (blocks > 0x7fffffffLL) return set_error(QFA_EUNSUPPORTED, "dout_normalise: too many elements for one launch");
+  dout_max_kernel<T, S><<<dim3(NORM_BLOCKS), dim3(256), 0, st>>>((const T *)dout, n8, (const S *)scale, ns, partials);
+  dout_scale_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, st>>>((const T *)dout, n8, partials, (_Float16 *)out, back);
+  return check_launch("qfa_dout_normalise");
+}
+
+int64_t dout_normalise_workspace_bytes() { return (int64_t)NORM_BLOCKS * 2 * sizeof(float); }
+
+int launch_dout_normalise(const void *dout, int dout_dtype, int64_t n, const void *scale, int scale_dtype, int64_t ns,
+                          float *partials, void *out, float *back, hipStream_t st) {
+  const bool s32 = scale_dtype == QFA_F32;
+  if (dout_dtype == QFA_BF16)
+    return s32 ? launch_dout_normalise_ts<__bf16, float>(dout, n, scale, ns, partials, out, back, st)
+               : launch_dout_normalise_ts<__bf16, _Float16>(dout, n, scale, ns, partials, out, back, st);
+  return s32 ? launch_dout_normalise_ts<_Float16, float>(dout, n, scale, ns, partials, out, back, st)
+             : launch_dout_normalise_ts<_Float16, _Float16>(dout, n, scale, ns, partials, out, back, st);
+}
+
 }  // namespace qfa

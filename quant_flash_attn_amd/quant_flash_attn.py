@@ -355,18 +355,30 @@ class QuantFlashAttention(torch.autograd.Function):
 
 
 def _normalised_dout(grad_output: torch.Tensor, kv_scale: torch.Tensor):
-    """(dO * 2^k as float16, 2^-k as a one-element float32 tensor) for the binary16 backward kernels.
+    """(dO * 2^k as float16, 2^-k as a one-element float32 tensor) for the binary16 backward kernels
+    (qfa_dout_normalise: two launches, nothing synchronises).
 
-    k puts the largest |dO| * 2^k * (largest key scale) at 8: 2^8 for |dO| when the key scales are of the usual size
-    (2^-5 for values of order one), higher when they are smaller and lower when they are larger, since the operands
+    k puts the largest |dO| * 2^k * (largest key scale) into (4, 8]: 2^8 for |dO| when the key scales are of the usual
+    size (2^-5 for values of order one), higher when they are smaller and lower when they are larger, since the operands
     the kernels form carry the key scale as a factor (ds * scale_j must neither sink into binary16's subnormals nor
-    leave its range); dO * 2^k itself stays below 2^14.  Everything is computed on the device."""
-    do32 = grad_output.to(torch.float32)
-    amax = do32.abs().amax().clamp_min(1e-30)
-    smax = kv_scale.to(torch.float32).abs().amax().clamp_min(1e-30)
-    k = torch.minimum(torch.floor(torch.log2(8.0 / (amax * smax))), torch.floor(torch.log2(16384.0 / amax)))
-    k = k.clamp_(-100.0, 100.0)
-    return (do32 * torch.exp2(k)).to(torch.float16), torch.exp2(-k)
+    leave its range); dO * 2^k itself stays at or below 2^14."""
+    _lib.require_gpu(grad_output, kv_scale)
+    if grad_output.dtype not in _IO_DTYPES:   # not what autograd hands over for a 16-bit output; bf16 keeps the range
+        grad_output = grad_output.to(torch.bfloat16)
+    grad_output = grad_output.contiguous()
+    if kv_scale.dtype not in (torch.float32, torch.float16):
+        kv_scale = kv_scale.to(torch.float32)
+    kv_scale = kv_scale.contiguous()
+    dev = grad_output.device
+    do16 = torch.empty(grad_output.shape, dtype=torch.float16, device=dev)
+    back = torch.empty(1, dtype=torch.float32, device=dev)
+    workspace = torch.empty(_lib.lib().qfa_dout_normalise_workspace_bytes(), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().qfa_dout_normalise(
+            grad_output.data_ptr(), _lib.DTYPE_CODE[grad_output.dtype], grad_output.numel(), kv_scale.data_ptr(),
+            _lib.DTYPE_CODE[kv_scale.dtype], kv_scale.numel(), workspace.data_ptr(), do16.data_ptr(), back.data_ptr(),
+            _lib.stream_of(grad_output)), "qfa_dout_normalise")
+    return do16, back
 
 
 def _legacy_operands(q, codes, scale, zp, io):

@@ -94,6 +94,20 @@ def test_argument_errors_need_no_gpu(qfa):
     assert skv_bwd(io=2) == -2 and b"QFA_F16" in L.qfa_last_error()
     assert skv_bwd(dkv=None) == -1 and b"null" in L.qfa_last_error()
     assert skv_bwd(gd=0) == -1 and b"grad_dtype" in L.qfa_last_error()
+    # the two small passes around the backward kernels
+    assert L.qfa_sum_grads(ok_ptr, None, ok_ptr, 2, 64, None) == -1 and b"null" in L.qfa_last_error()
+    assert L.qfa_sum_grads(ok_ptr, ok_ptr, ok_ptr, 0, 64, None) == -1 and b"dtype" in L.qfa_last_error()
+    assert L.qfa_sum_grads(ok_ptr, ok_ptr, ok_ptr, 2, 12, None) == -1 and b"multiple of 8" in L.qfa_last_error()
+    assert L.qfa_sum_grads(ok_ptr, ok_ptr + 2, ok_ptr, 2, 64, None) == -1 and b"aligned" in L.qfa_last_error()
+    assert L.qfa_dout_normalise_workspace_bytes() > 0
+    def norm(dout=ok_ptr, dt=1, n=64, sdt=0, ns=5, ws=ok_ptr):
+        return L.qfa_dout_normalise(dout, dt, n, ok_ptr, sdt, ns, ws, ok_ptr, ok_ptr, None)
+    assert norm(ws=None) == -1 and b"null" in L.qfa_last_error()
+    assert norm(dt=0) == -1 and b"dout_dtype" in L.qfa_last_error()
+    assert norm(sdt=2) == -1 and b"scale_dtype" in L.qfa_last_error()
+    assert norm(n=20) == -1 and b"multiple of 8" in L.qfa_last_error()
+    assert norm(ns=0) == -1 and b"n_scale" in L.qfa_last_error()
+    assert norm(dout=ok_ptr + 4) == -1 and b"aligned" in L.qfa_last_error()
 
 
 def test_cpu_tensors_are_refused_not_emulated(qfa):

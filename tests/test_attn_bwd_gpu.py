@@ -287,6 +287,34 @@ def test_reference_entry_point_shared_kv(qfa, Z, H, Nq, Nkv, D):
     assert_close("dKV", kvg.grad.cpu(), dkv_ref, scaled=True, spread=nkv)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n", [16, 64 * 1024 - 8, 3 * 1024 * 1024 + 40])
+def test_sum_grads_is_the_fp32_sum_rounded_once(qfa, dtype, n):
+    """dkv = dK + dV of the reference's entry point (quant_flash_attn.py:161) through the C-ABI: both addends
+    widened to fp32, added, rounded once to the 16-bit format -- bit for bit, also in place (out = a), with values
+    that cancel, overflow the format and non-finite ones."""
+    from quant_flash_attn_amd import _lib
+    g = torch.Generator().manual_seed(n)
+    a = (torch.randn(n, generator=g) * 8).to(dtype)
+    b = (torch.randn(n, generator=g) * 8).to(dtype)
+    b[::7] = -a[::7]
+    big = torch.finfo(dtype).max
+    special = torch.tensor([big, big, -big, float("inf"), float("nan"), 0.0, -0.0, 2.0 ** -20], dtype=dtype)
+    a[:8], b[:8] = special, special.flip(0)
+    a[8:16], b[8:16] = special, special
+    a, b = a.to(DEV), b.to(DEV)
+    want = (a.float() + b.float()).to(dtype)
+    out = torch.empty_like(a)
+    code = _lib.DTYPE_CODE[dtype]
+    _lib.check(_lib.lib().qfa_sum_grads(a.data_ptr(), b.data_ptr(), out.data_ptr(), code, n, _lib.stream_of(a)), "sum")
+    _lib.check(_lib.lib().qfa_sum_grads(a.data_ptr(), b.data_ptr(), a.data_ptr(), code, n, _lib.stream_of(a)), "sum")
+    torch.cuda.synchronize()
+    for got in (out, a):
+        assert torch.equal(got.view(torch.int16)[~want.isnan()], want.view(torch.int16)[~want.isnan()])
+        assert torch.equal(got.isnan(), want.isnan())
+    assert _lib.lib().qfa_sum_grads(a.data_ptr(), b.data_ptr(), out.data_ptr(), code, 12, _lib.stream_of(a)) != 0
+
+
 def test_graph_capture_and_replay(qfa):
     """The whole step (both quantizers, forward, backward) captured into a HIP graph: every entry point
     only enqueues kernels on the caller's stream (no allocation, no memset, no synchronisation inside

@@ -177,6 +177,40 @@ def test_shared_kv_entry_point_fp16_small_gradients(qfa, do_scale, kv_scale, Nq)
     assert_close("dKV", kvd.grad.cpu().double() / do_scale, r16(dkv_ref) / do_scale, scaled=True, rel=REL_TOL[torch.float16])
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("sdtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("do_scale,kv_scale", [(1.0, 2.0 ** -5), (2.0 ** -14, 2.0 ** -5), (2.0 ** -20, 2.0 ** -11), (300.0, 2.0 ** -5),
+                                               (1.0, 40.0), (3.0, 2.0 ** -16), (0.0, 1.0)])
+def test_dout_normalisation_through_the_c_abi(qfa, dtype, sdtype, do_scale, kv_scale):
+    """qfa_dout_normalise: out = binary16(dO * 2^k) and back = 2^-k, with k the largest integer such that
+    max|dO| * 2^k * max|scale| <= 8 and max|dO| * 2^k <= 2^14 (the product of the two maxima taken in fp32) --
+    computed here with exact integer arithmetic on the exponents; out and back bit for bit."""
+    import numpy as np
+    from quant_flash_attn_amd import _lib
+    from quant_flash_attn_amd.quant_flash_attn import _normalised_dout
+    g = torch.Generator().manual_seed(3)
+    do = (torch.randn(3, 5, 17, 64, generator=g) * do_scale).to(dtype)
+    do[1, 2, 3, 4] = do_scale * 4.0       # the maximum, an exact power of two when do_scale is one
+    sc = (torch.rand(3, 5, 1000, generator=g) * kv_scale).to(sdtype)
+    if do_scale == 1.0 and kv_scale == 2.0 ** -5:
+        sc[0, 0, 0] = 2.0 ** -5           # product of the maxima exactly 2^-3: k = 6, not 5
+    amax = np.float32(max(float(do.float().abs().max()), 1e-30))
+    smax = np.float32(max(float(sc.float().abs().max()), 1e-30))
+    def floor_log2_quot(ce, y):           # floor(log2(2^ce / y)) for a positive float y
+        m, e = math.frexp(float(y))       # y = m * 2^e, m in [0.5, 1)
+        return ce - e + (1 if m == 0.5 else 0) if y > 0 else 10 ** 6
+    k = min(floor_log2_quot(3, np.float32(amax * smax)), floor_log2_quot(14, amax))
+    k = max(-100, min(100, k))
+    do16, back = _normalised_dout(do.to(DEV), sc.to(DEV))
+    assert do16.dtype == torch.float16 and do16.shape == do.shape and back.dtype == torch.float32
+    assert float(back.cpu()) == 2.0 ** -k, (float(back.cpu()), k)
+    want = (do.double() * 2.0 ** k).to(torch.float16)
+    assert torch.equal(do16.cpu().view(torch.int16), want.view(torch.int16))
+    if do_scale > 0:
+        top = float(amax) * 2.0 ** k
+        assert top <= 2.0 ** 14 and (top * float(smax) > 4.0 * (1 - 1e-6) or top > 2.0 ** 13)
+
+
 def test_shared_kv_entry_point_long_query_block(qfa):
     """97 queries (a reference test shape, test_accuracy.py:44): the forward splits them over workgroups
     of 16, the backward runs its dQ and dKV kernels."""
