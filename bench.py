@@ -42,10 +42,10 @@ PEAK_INT8_TOPS = 5000.0
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per forward launch at the headline configuration, measured with rocprofv3 --pmc:
-# FETCH_SIZE 199 083 KiB x 2.000 (calibration: 256 MiB copy reads 131 085) + WRITE_SIZE 133 120 KiB x 1.000
+# FETCH_SIZE 204 131 KiB x 2.000 (calibration: 256 MiB copy reads 131 086) + WRITE_SIZE 133 120 KiB x 1.000
 # (profiles/kernels_B4_H32_N4096_D128_causal_bf16.md); algorithmic bytes are 395 MiB -- the causal dispatch
 # order keeps four heads in flight per XCD, more than its L2 holds, and the re-reads show up here
-FWD_TRAFFIC_BYTES = (199083 * 2 + 133120) * 1024
+FWD_TRAFFIC_BYTES = (204131 * 2 + 133120) * 1024
 
 
 def flops_fwd(B, H, Nq, Nk, D, causal):
