@@ -222,8 +222,8 @@ int qfa_bench_qk_stage(const int8_t *qc, const float *sq, const int8_t *zq, cons
                        int64_t sob, int64_t soh, int64_t son, float sm_scale, int causal, void *stream);
 
 /*
- * out = dout * 2^k as binary16 and back[0] = 2^-k, for a dense 16-bit dout of n elements (n a multiple of 8, dout and
- * out 16-byte aligned) and the n_scale per-token scales of the shared K = V tensor (QFA_F32 or QFA_F16).
+ * out = dout * 2^k as binary16 and back[0] = 2^-k, for a dense 16-bit dout of n elements (n a multiple of 8) and the
+ * n_scale per-token scales of the shared K = V tensor (QFA_F32 or QFA_F16); dout, kv_scale and out 16-byte aligned.
  * qfa_attn_bwd_shared_kv computes in binary16 and forms sm_scale * p * (dP - delta) * scale_j as a matrix operand;
  * dQ and dKV are linear in dO, so callers hand it this scaled dO and pass `back` as grad_scale.  k is the largest
  * integer with  max|dout| * 2^k * max|scale| <= 8  and  max|dout| * 2^k <= 2^14  (within [-100, 100]), found on the

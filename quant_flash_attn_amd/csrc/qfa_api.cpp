@@ -312,7 +312,8 @@ int qfa_dout_normalise(const void *dout, int dout_dtype, int64_t n, const void *
   if (scale_dtype != QFA_F32 && scale_dtype != QFA_F16) return set_error(QFA_EINVAL, "dout_normalise: scale_dtype must be QFA_F32 or QFA_F16");
   if (n <= 0 || n % 8 != 0) return set_error(QFA_EINVAL, "dout_normalise: the element count must be a positive multiple of 8");
   if (n_scale <= 0) return set_error(QFA_EINVAL, "dout_normalise: n_scale must be positive");
-  if (!aligned16(dout) || !aligned16(out)) return set_error(QFA_EINVAL, "dout_normalise: dout and out must be 16-byte aligned");
+  if (!aligned16(dout) || !aligned16(out) || !aligned16(kv_scale))
+    return set_error(QFA_EINVAL, "dout_normalise: dout, kv_scale and out must be 16-byte aligned");
   return launch_dout_normalise(dout, dout_dtype, n, kv_scale, scale_dtype, n_scale, static_cast<float *>(workspace), out, back,
                                (hipStream_t)stream);
 }

@@ -449,12 +449,22 @@ int launch_skv_bwd(const SkvAttnArgs &x, hipStream_t st) {
 // max|dO| * 2^k at or below 2^14, so that neither ordinary small gradients sink into binary16's subnormals nor large
 // key scales leave its range.  Two launches, no atomics: every block of the first writes its two partial maxima,
 // every block of the second reduces all of them again (a few KB out of the L2) before it scales its share.
-constexpr int NORM_BLOCKS = 512;   // blocks of the first launch = pairs of floats in the partials buffer
+constexpr int NORM_BLOCKS = 2048;   // blocks of the first launch = pairs of floats in the partials buffer
 
 template <typename T> __device__ __forceinline__ float max_abs8(const u32x4 w, float m) {
 #pragma unroll
   for (int e = 0; e < 4; ++e) m = fmaxf(m, fmaxf(fabsf(lo_to_f32<T>(w[e])), fabsf(hi_to_f32<T>(w[e]))));
   return m;
+}
+// largest magnitude of the 16 bytes of scales a thread loads at a time
+template <typename S> __device__ __forceinline__ float max_abs_chunk(const u32x4 w, float m) {
+  if constexpr (sizeof(S) == 2) {
+    return max_abs8<S>(w, m);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) m = fmaxf(m, fabsf(__builtin_bit_cast(float, w[e])));
+    return m;
+  }
 }
 __device__ __forceinline__ float block_max_256(float m, float *red) {
   for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
@@ -470,14 +480,16 @@ __device__ __forceinline__ int floor_log2_quot(int ce, float y) {
   return ce - e - ((b & 0x7fffffu) != 0 ? 1 : 0);
 }
 
+// 16 bytes per thread and trip for both vectors (the scales' last ns % (16 / sizeof(S)) elements one by one)
 template <typename T, typename S>
 __global__ __launch_bounds__(256) void dout_max_kernel(const T *dout, int64_t n8, const S *scale, int64_t ns, float *partials) {
   __shared__ float red[4];
+  constexpr int EPC = 16 / sizeof(S);
+  const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x, nth = (int64_t)NORM_BLOCKS * 256, nsc = ns / EPC;
   float m = 0.f, ms = 0.f;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)NORM_BLOCKS * 256)
-    m = max_abs8<T>(reinterpret_cast<const u32x4 *>(dout)[i], m);
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < ns; i += (int64_t)NORM_BLOCKS * 256)
-    ms = fmaxf(ms, fabsf((float)scale[i]));
+  for (int64_t i = tid; i < n8; i += nth) m = max_abs8<T>(reinterpret_cast<const u32x4 *>(dout)[i], m);
+  for (int64_t i = tid; i < nsc; i += nth) ms = max_abs_chunk<S>(reinterpret_cast<const u32x4 *>(scale)[i], ms);
+  if (tid < ns - nsc * EPC) ms = fmaxf(ms, fabsf((float)scale[nsc * EPC + tid]));
   m = block_max_256(m, red);
   ms = block_max_256(ms, red);
   if (threadIdx.x == 0) {

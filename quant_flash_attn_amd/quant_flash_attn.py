@@ -369,6 +369,8 @@ def _normalised_dout(grad_output: torch.Tensor, kv_scale: torch.Tensor):
     if kv_scale.dtype not in (torch.float32, torch.float16):
         kv_scale = kv_scale.to(torch.float32)
     kv_scale = kv_scale.contiguous()
+    if kv_scale.data_ptr() % 16:   # a view that starts inside an allocation
+        kv_scale = kv_scale.clone()
     dev = grad_output.device
     do16 = torch.empty(grad_output.shape, dtype=torch.float16, device=dev)
     back = torch.empty(1, dtype=torch.float32, device=dev)

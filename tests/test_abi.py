@@ -108,6 +108,7 @@ def test_argument_errors_need_no_gpu(qfa):
     assert norm(n=20) == -1 and b"multiple of 8" in L.qfa_last_error()
     assert norm(ns=0) == -1 and b"n_scale" in L.qfa_last_error()
     assert norm(dout=ok_ptr + 4) == -1 and b"aligned" in L.qfa_last_error()
+    assert L.qfa_dout_normalise(ok_ptr, 1, 64, ok_ptr + 2, 1, 5, ok_ptr, ok_ptr, ok_ptr, None) == -1 and b"aligned" in L.qfa_last_error()
 
 
 def test_cpu_tensors_are_refused_not_emulated(qfa):

@@ -191,7 +191,7 @@ def test_dout_normalisation_through_the_c_abi(qfa, dtype, sdtype, do_scale, kv_s
     g = torch.Generator().manual_seed(3)
     do = (torch.randn(3, 5, 17, 64, generator=g) * do_scale).to(dtype)
     do[1, 2, 3, 4] = do_scale * 4.0       # the maximum, an exact power of two when do_scale is one
-    sc = (torch.rand(3, 5, 1000, generator=g) * kv_scale).to(sdtype)
+    sc = (torch.rand(3, 5, 1003, generator=g) * kv_scale).to(sdtype)     # 15 045 scales: a tail after the 16-byte chunks
     if do_scale == 1.0 and kv_scale == 2.0 ** -5:
         sc[0, 0, 0] = 2.0 ** -5           # product of the maxima exactly 2^-3: k = 6, not 5
     amax = np.float32(max(float(do.float().abs().max()), 1e-30))
@@ -202,6 +202,9 @@ def test_dout_normalisation_through_the_c_abi(qfa, dtype, sdtype, do_scale, kv_s
     k = min(floor_log2_quot(3, np.float32(amax * smax)), floor_log2_quot(14, amax))
     k = max(-100, min(100, k))
     do16, back = _normalised_dout(do.to(DEV), sc.to(DEV))
+    pad = torch.cat([sc.flatten()[:1], sc.flatten()]).to(DEV)      # the same scales as a view that is not 16-byte aligned
+    do16_b, back_b = _normalised_dout(do.to(DEV), pad[1:])
+    assert torch.equal(do16_b, do16) and torch.equal(back_b, back)
     assert do16.dtype == torch.float16 and do16.shape == do.shape and back.dtype == torch.float32
     assert float(back.cpu()) == 2.0 ** -k, (float(back.cpu()), k)
     want = (do.double() * 2.0 ** k).to(torch.float16)
