@@ -196,6 +196,10 @@ def main():
     extra["quant_ms_per_tensor"] = round(ms_quant, 4)
     extra["quant_GBps"] = round(quant_bytes / (ms_quant * 1e-3) / 1e9, 1)
     extra["quant_frac_hbm_peak"] = round(quant_bytes / (ms_quant * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)
+    # the step's form: queries and keys in one launch (twice the bytes)
+    ms_pair = time_events(lambda: qfa.quantize_pair_for_attention(q, k), 50, 10)
+    extra["quant_pair_ms"] = round(ms_pair, 4)
+    extra["quant_pair_GBps"] = round(2 * quant_bytes / (ms_pair * 1e-3) / 1e9, 1)
     ms_fwd_only = time_events(lambda: qfa.attn_fwd_quantized(qq, kq, v, causal, sm), args.steps, 5)
     extra["fwd_kernel_ms"] = round(ms_fwd_only, 4)
     extra["fwd_kernel_tflops"] = round(F_fwd / (ms_fwd_only * 1e-3) / 1e12, 2)
