@@ -24,9 +24,10 @@
 // is an integer below 2^24, hence exact in fp32.  Then one multiply by the key scale; the query
 // scale, sm_scale and log2(e) are folded into the exp2 argument.
 //
-// What bounds the kernel is the issue rate of the vector pipe (every vector instruction takes about 4.5
-// cycles of it with two waves per SIMD and an MFMA about twice that, whatever else overlaps), so the design goal is
-// the smallest number of vector instructions per score:
+// With two waves per SIMD (64 O accumulators per wave leave no room for a third at head_dim 128) every vector
+// instruction takes about 4.5 cycles of issue and an MFMA about twice that, whatever else overlaps, and no pipe is
+// saturated (matrix 52 %, vector 53 % busy at the headline size): the time is the length of a wave's instruction
+// stream plus the latency two waves cannot cover.  So the design goal is the smallest number of instructions per score:
 //  * the reference maximum is only moved (and O rescaled) when it has to be (any reference gives the
 //    same O after the final division): the masked loop moves it when a row exceeds it by more than
 //    2^8, the pipelined loop takes no maximum at all and watches the running sum of the probabilities
