@@ -94,6 +94,16 @@ def test_argument_errors_need_no_gpu(qfa):
     assert skv_bwd(io=2) == -2 and b"QFA_F16" in L.qfa_last_error()
     assert skv_bwd(dkv=None) == -1 and b"null" in L.qfa_last_error()
     assert skv_bwd(gd=0) == -1 and b"grad_dtype" in L.qfa_last_error()
+    # queries and keys in one launch: the same checks per tensor
+    def pair(x1=ok_ptr, dt=2, N1=8, D=64, sx1=(512, 512, 64)):
+        return L.qfa_quant_per_token_pair(ok_ptr, x1, dt, *([ok_ptr] * 8), 1, 1, 8, N1, D, 512, 512, 64, *sx1,
+                                          512, 512, 64, 512, 512, 64, None)
+    assert pair(x1=None) == -1 and b"null" in L.qfa_last_error()
+    assert pair(dt=9) == -1 and b"x_dtype" in L.qfa_last_error()
+    assert pair(N1=0) == -1 and b"positive" in L.qfa_last_error()
+    assert pair(D=44) == -2 and b"head_dim" in L.qfa_last_error()
+    assert pair(x1=ok_ptr + 2) == -1 and b"aligned" in L.qfa_last_error()
+    assert pair(sx1=(512, 512, 60)) == -1 and b"strides" in L.qfa_last_error()
     # the two small passes around the backward kernels
     assert L.qfa_sum_grads(ok_ptr, None, ok_ptr, 2, 64, None) == -1 and b"null" in L.qfa_last_error()
     assert L.qfa_sum_grads(ok_ptr, ok_ptr, ok_ptr, 0, 64, None) == -1 and b"dtype" in L.qfa_last_error()
